@@ -1,0 +1,49 @@
+// Shared device helpers for the gfx950 kernels: element types, conversions, wave and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16;
+
+#define WAVE 64
+
+// Error codes returned by every extern "C" entry point (0 = launched).
+#define MS_OK 0
+#define MS_BAD_ARG 1
+#define MS_UNSUPPORTED 2
+#define MS_LAUNCH_FAILED 3
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16 x) { return static_cast<float>(x); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float x) { return static_cast<bf16>(x); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+  return v;
+}
+
+// Sum over a block of NT threads (NT a multiple of 64, at most 1024). `red` holds NT / 64 floats.
+// Every thread receives the total; the order of additions is fixed by NT alone.
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / WAVE; ++i) total += red[i];
+  return total;
+}
+
+static inline int launch_status() { return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED; }

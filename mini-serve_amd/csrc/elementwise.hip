@@ -1,0 +1,187 @@
+// Embedding gather, RMSNorm, gated activation, casts, and the fused per-head norm + rotation +
+// cache store. All arithmetic is float32; bfloat16 appears only as a storage type and each
+// result is rounded once.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// out[t, :] = float(table[ids[t], :])
+template <typename TW>
+__global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const TW* src = table + (size_t)ids[t] * width;
+  float* dst = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+extern "C" int ms_embed(const int* ids, const void* table, int table_is_bf16, float* out, int tokens, int width, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (width <= 0) return MS_BAD_ARG;
+  if (table_is_bf16)
+    embed_kernel<bf16><<<tokens, 256, 0, st>>>(ids, (const bf16*)table, out, width);
+  else
+    embed_kernel<float><<<tokens, 256, 0, st>>>(ids, (const float*)table, out, width);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// y[r, :] = w * x[row(r), :] * rsqrt(mean(x^2) + eps), float32 throughout, rounded once.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w, TO* __restrict__ y,
+                               const int* __restrict__ rows, int width, float eps) {
+  __shared__ float red[256 / WAVE];
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = src[i];
+    ss += v * v;
+  }
+  ss = block_sum<256>(ss, red);
+  const float rstd = rsqrtf(ss / (float)width + eps);
+  TO* dst = y + (size_t)r * width;
+  for (int i = threadIdx.x; i < width; i += 256) dst[i] = from_f32<TO>(src[i] * rstd * to_f32(w[i]));
+}
+
+extern "C" int ms_rmsnorm(const float* x, const void* w, int w_is_bf16, void* y, int y_is_bf16, const int* rows,
+                          int n_rows, int width, float eps, hipStream_t st) {
+  if (n_rows <= 0) return MS_OK;
+  if (width <= 0) return MS_BAD_ARG;
+#define LAUNCH(TW, TO) rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, st>>>(x, (const TW*)w, (TO*)y, rows, width, eps)
+  if (w_is_bf16 && y_is_bf16) LAUNCH(bf16, bf16);
+  else if (w_is_bf16) LAUNCH(bf16, float);
+  else if (y_is_bf16) LAUNCH(float, bf16);
+  else LAUNCH(float, float);
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i]
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= inter) return;
+  const float g = to_f32(gu[(size_t)t * 2 * inter + i]);
+  const float u = to_f32(gu[(size_t)t * 2 * inter + inter + i]);
+  out[(size_t)t * inter + i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int ms_silu_mul(const void* gu, void* out, int is_bf16, int tokens, int inter, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (inter <= 0 || tokens > 65535) return MS_BAD_ARG;
+  dim3 grid((inter + 255) / 256, tokens);
+  if (is_bf16) silu_mul_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter);
+  else silu_mul_kernel<float><<<grid, 256, 0, st>>>((const float*)gu, (float*)out, inter);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<TO>(to_f32(in[i]));
+}
+
+extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf16, long long n, hipStream_t st) {
+  if (n <= 0) return MS_OK;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (in_is_bf16 && !out_is_bf16) cast_kernel<bf16, float><<<blocks, 256, 0, st>>>((const bf16*)in, (float*)out, (size_t)n);
+  else if (!in_is_bf16 && out_is_bf16) cast_kernel<float, bf16><<<blocks, 256, 0, st>>>((const float*)in, (bf16*)out, (size_t)n);
+  else return MS_BAD_ARG;
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// One wave per (token, head slot). Head slots [0, Hq) are query heads, [Hq, Hq+Hkv) key heads,
+// [Hq+Hkv, Hq+2Hkv) value heads of the token's row in qkv [tokens, (Hq + 2 Hkv) * D].
+//   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
+//         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j];
+//   q is written back in place; k and v go to the cache page of the token's slot
+//   (cache layout [pages, Hkv, page_size, D]; slot = page * page_size + offset).
+// With slots == nullptr only the query heads are processed (the entry reads another entry's cache).
+#define MAX_HEAD_DIM 256
+template <typename T, typename TW>
+__global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const int* __restrict__ slots,
+                                          const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
+                                          const float* __restrict__ inv_freq, int rot, T* __restrict__ kc,
+                                          T* __restrict__ vc, int Hq, int Hkv, int D, int page_size) {
+  __shared__ float buf[MAX_HEAD_DIM];
+  const int t = blockIdx.x, hs = blockIdx.y, lane = threadIdx.x;
+  const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);
+  T* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + hs) * D;
+  constexpr int PER = MAX_HEAD_DIM / WAVE;
+  float x[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + i * WAVE;
+    x[i] = e < D ? to_f32(src[e]) : 0.f;
+    ss += x[i] * x[i];
+  }
+  T* dst = src;
+  if (kind != 0) {
+    const int s = slots[t];
+    const int kvh = kind == 1 ? hs - Hq : hs - Hq - Hkv;
+    T* base = kind == 1 ? kc : vc;
+    dst = base + (((size_t)(s / page_size) * Hkv + kvh) * page_size + (s % page_size)) * D;
+  }
+  if (kind != 2) {
+    const TW* w = kind == 0 ? qw : kw;
+    if (w != nullptr) {
+      ss = wave_sum(ss);
+      const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = lane + i * WAVE;
+        if (e < D) x[i] = x[i] * rstd * to_f32(w[e]);
+      }
+    }
+    if (rot > 0) {
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = lane + i * WAVE;
+        if (e < D) buf[e] = x[i];
+      }
+      __syncthreads();
+      const int half = rot / 2;
+      const float p = (float)pos[t];
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = lane + i * WAVE;
+        if (e < rot) {
+          const int j = e < half ? e : e - half;
+          float sn, cs;
+          sincosf(p * inv_freq[j], &sn, &cs);
+          x[i] = e < half ? x[i] * cs - buf[e + half] * sn : x[i] * cs + buf[e - half] * sn;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + i * WAVE;
+    if (e < D) dst[e] = from_f32<T>(x[i]);
+  }
+}
+
+extern "C" int ms_qk_norm_rope_store(void* qkv, int is_bf16, const int* pos, const int* slots, const void* qw,
+                                     const void* kw, int w_is_bf16, float eps, const float* inv_freq, int rot, void* kc,
+                                     void* vc, int tokens, int Hq, int Hkv, int D, int page_size, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (D <= 0 || D > MAX_HEAD_DIM || rot < 0 || rot > D || (rot & 1) || Hq <= 0 || Hkv <= 0 || page_size <= 0) return MS_BAD_ARG;
+  if ((qw == nullptr) != (kw == nullptr)) return MS_BAD_ARG;
+  if (rot > 0 && inv_freq == nullptr) return MS_BAD_ARG;
+  const int heads = slots ? Hq + 2 * Hkv : Hq;
+  if (heads > 65535) return MS_BAD_ARG;
+  dim3 grid(tokens, heads);
+#define LAUNCH(T, TW)                                                                                              \
+  qk_norm_rope_store_kernel<T, TW><<<grid, WAVE, 0, st>>>((T*)qkv, pos, slots, (const TW*)qw, (const TW*)kw, eps, \
+                                                           inv_freq, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size)
+  if (is_bf16 && w_is_bf16) LAUNCH(bf16, bf16);
+  else if (is_bf16) LAUNCH(bf16, float);
+  else if (w_is_bf16) LAUNCH(float, bf16);
+  else LAUNCH(float, float);
+#undef LAUNCH
+  return launch_status();
+}

@@ -1,0 +1,239 @@
+// bfloat16 matrix products C[M, N] = X[M, K] * W[N, K]^T on the gfx950 matrix cores
+// (v_mfma_f32_16x16x32_bf16, float32 accumulation), in two shapes:
+//
+//  * tile kernel   (prefill, M large): BM x BN macro-tiles staged through LDS in K-slabs of 64 with a
+//                  register prefetch of the next slab; 4 waves in a 2 x 2 grid of wave tiles.
+//  * skinny kernel (decode, M <= 64): pure weight streaming. A wave owns 16 weight rows and walks
+//                  all of K with 32-byte loads per lane; the few activation rows come from LDS.
+//
+// Operand roles: the weight rows are the MFMA's A operand (its row index i = n) and the activation
+// rows the B operand (column index j = m), so a lane ends up with four consecutive n of one m and
+// stores them as one vector.
+//
+// Layout of v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16):
+//   A operand: 8 values A[i = r][k = 8 g .. 8 g + 7]     B operand: 8 values B[k = 8 g .. 8 g + 7][j = r]
+//   result:    4 values D[i = 4 g + 0..3][j = r]
+// Any permutation of k that is the same for both operands leaves the result unchanged; the skinny
+// kernel uses that to let a lane load 16 consecutive k at once.
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+union Chunk {  // 8 bf16 = 16 bytes
+  uint4 u;
+  bf16x8 v;
+  bf16 e[8];
+};
+
+// 8 consecutive k of one row, zero where the row or k is out of range.
+__device__ __forceinline__ Chunk load_chunk(const bf16* __restrict__ base, int row, int rows, int k, int K, size_t ld, bool vec) {
+  Chunk c;
+  if (row < rows && vec && k + 8 <= K) {
+    c.u = *reinterpret_cast<const uint4*>(base + (size_t)row * ld + k);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c.e[i] = (row < rows && k + i < K) ? base[(size_t)row * ld + k + i] : static_cast<bf16>(0.f);
+  }
+  return c;
+}
+
+// Store four consecutive n of row m. mode 0: bf16, 1: float, 2: float +=.
+__device__ __forceinline__ void store4(void* __restrict__ C, int mode, int m, int n, int M, int N, int ldc, floatx4 a, bool vec_ok) {
+  if (m >= M || n >= N) return;
+  const size_t at = (size_t)m * ldc + n;
+  if (vec_ok && n + 3 < N) {
+    if (mode == 0) {
+      union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.e[i] = static_cast<bf16>(a[i]);
+      *reinterpret_cast<uint2*>((bf16*)C + at) = o.u;
+    } else if (mode == 1) {
+      *reinterpret_cast<float4*>((float*)C + at) = make_float4(a[0], a[1], a[2], a[3]);
+    } else {
+      float4 c = *reinterpret_cast<float4*>((float*)C + at);
+      c.x += a[0]; c.y += a[1]; c.z += a[2]; c.w += a[3];
+      *reinterpret_cast<float4*>((float*)C + at) = c;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (n + i >= N) break;
+      if (mode == 0) ((bf16*)C)[at + i] = static_cast<bf16>(a[i]);
+      else if (mode == 1) ((float*)C)[at + i] = a[i];
+      else ((float*)C)[at + i] += a[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tile kernel.
+#define BK 64
+#define LDS_STRIDE (BK + 8)  // bf16 elements per LDS row: 144 bytes, keeps 16-byte alignment
+
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                             void* __restrict__ C, int mode, int M, int N, int K,
+                                                             int ldx, int ldc) {
+  constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
+  constexpr int FM = WM / 16, FN = WN / 16;    // 16 x 16 fragments per wave tile
+  constexpr int XCH = BM * (BK / 8) / 256;     // 16-byte chunks per thread per slab
+  constexpr int WCH = BN * (BK / 8) / 256;
+  __shared__ __attribute__((aligned(16))) bf16 xs[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16 ws[BN * LDS_STRIDE];
+
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
+  const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
+
+  floatx4 acc[FN][FM];
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  Chunk xr[XCH], wr[WCH];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int c = tid + i * 256;
+      xr[i] = load_chunk(X, m0 + c / (BK / 8), M, k0 + (c % (BK / 8)) * 8, K, ldx, vecx);
+    }
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) {
+      const int c = tid + i * 256;
+      wr[i] = load_chunk(W, n0 + c / (BK / 8), N, k0 + (c % (BK / 8)) * 8, K, K, vecw);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int c = tid + i * 256;
+      *reinterpret_cast<uint4*>(&xs[(c / (BK / 8)) * LDS_STRIDE + (c % (BK / 8)) * 8]) = xr[i].u;
+    }
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) {
+      const int c = tid + i * 256;
+      *reinterpret_cast<uint4*>(&ws[(c / (BK / 8)) * LDS_STRIDE + (c % (BK / 8)) * 8]) = wr[i].u;
+    }
+  };
+
+  fetch(0);
+  stash();
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    const bool more = k0 + BK < K;
+    if (more) fetch(k0 + BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 32) {
+      bf16x8 wf[FN], xf[FM];
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+        wf[i] = *reinterpret_cast<const bf16x8*>(&ws[(wn + i * 16 + r) * LDS_STRIDE + kk + g * 8]);
+#pragma unroll
+      for (int j = 0; j < FM; ++j)
+        xf[j] = *reinterpret_cast<const bf16x8*>(&xs[(wm + j * 16 + r) * LDS_STRIDE + kk + g * 8]);
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+
+  const bool vec_store = (ldc % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j)
+      store4(C, mode, m0 + wm + j * 16 + r, n0 + wn + i * 16 + g * 4, M, N, ldc, acc[i][j], vec_store);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Skinny kernel: M <= 16 * MB rows of X. Block = 4 waves = 64 weight rows. K is walked in slabs of
+// KS; the X slab is staged in LDS once per block and shared by its waves.
+#define KS 256
+#define XS_STRIDE (KS + 8)
+
+template <int MB>
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                               void* __restrict__ C, int mode, int M, int N, int K,
+                                                               int ldx, int ldc) {
+  __shared__ __attribute__((aligned(16))) bf16 xs[MB * 16 * XS_STRIDE];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int nb = blockIdx.x * 64 + wave * 16;
+  const int n = nb + r;
+  const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
+
+  floatx4 acc[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int ks = 0; ks < K; ks += KS) {
+    __syncthreads();
+    // X slab [MB * 16][KS] into LDS, 16-byte chunks.
+    for (int c = tid; c < MB * 16 * (KS / 8); c += 256) {
+      const int m = c / (KS / 8), kc = (c % (KS / 8)) * 8;
+      const Chunk v = load_chunk(X, m, M, ks + kc, K, ldx, vecx);
+      *reinterpret_cast<uint4*>(&xs[m * XS_STRIDE + kc]) = v.u;
+    }
+    // This lane's weights of the slab: per block of 64 k, 16 consecutive k at offset 16 g.
+    Chunk w[KS / 64][2];
+#pragma unroll
+    for (int b = 0; b < KS / 64; ++b) {
+      const int k = ks + b * 64 + g * 16;
+      w[b][0] = load_chunk(W, n, N, k, K, K, vecw);
+      w[b][1] = load_chunk(W, n, N, k + 8, K, K, vecw);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < KS / 64; ++b) {
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const bf16* xp = &xs[(i * 16 + r) * XS_STRIDE + b * 64 + g * 16];
+        const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp);
+        const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + 8);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[b][0].v, x0, acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[b][1].v, x1, acc[i], 0, 0, 0);
+      }
+    }
+  }
+  const bool vec_store = (ldc % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < MB; ++i) store4(C, mode, i * 16 + r, nb + g * 4, M, N, ldc, acc[i], vec_store);
+}
+
+// mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
+extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,
+                            hipStream_t st) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (K <= 0 || ldx < K || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
+  const bf16* x = (const bf16*)X;
+  const bf16* w = (const bf16*)W;
+  if (M <= 64) {
+    dim3 grid((N + 63) / 64);
+    if (M <= 16) gemm_bf16_skinny_kernel<1><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+    else if (M <= 32) gemm_bf16_skinny_kernel<2><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+    else gemm_bf16_skinny_kernel<4><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+    return launch_status();
+  }
+  // Large tiles when they still give every CU work; small tiles otherwise.
+  const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (big >= 256) {
+    dim3 grid((N + 127) / 128, (M + 127) / 128);
+    if (grid.y > 65535) return MS_BAD_ARG;
+    gemm_bf16_tile_kernel<128, 128><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+  } else {
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    if (grid.y > 65535) return MS_BAD_ARG;
+    gemm_bf16_tile_kernel<64, 64><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+  }
+  return launch_status();
+}

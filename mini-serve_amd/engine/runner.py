@@ -1,0 +1,118 @@
+"""The model runner: owns the model, the cache manager and the pool, and offers the one step
+function every caller goes through (the scheduler's engine loop, trace replay, the benchmark).
+
+``step(rows)`` runs only the tokens it is given, as one batch, from the cache that earlier steps
+left, and returns float32 logits at the wanted places. It generalises the reference's
+``ModelRunner.forward`` (last new token of every row, miniserve/engine/model_runner.py:220-261) and
+``forward_tokens`` (every new position, :279-307).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..cache.allocator import OutOfBlocks
+from ..cache.manager import CacheLayout, CacheManager, RequestCache
+from ..cache.pool import KVPool
+from ..parts.model import DecoderModel
+from .batch import BatchBuilder, StepRow
+
+DEFAULT_PAGE_SIZE = 16
+
+
+class ModelRunner:
+    def __init__(
+        self,
+        model: DecoderModel,
+        page_size: int = DEFAULT_PAGE_SIZE,
+        kv_pool_tokens: int | None = None,
+        kv_mem_fraction: float = 0.9,
+        max_running: int = 64,
+        max_step_tokens: int | None = None,
+        allocator_class=None,
+    ):
+        """``kv_pool_tokens``: exact pool size in tokens (rounded down to whole pages; an error if
+        it holds no page or does not fit, never clipped; miniserve/engine/model_runner.py:99-108);
+        default: what ``kv_mem_fraction`` of the free memory holds after a reserve for activations.
+        ``max_step_tokens``: most tokens one step carries (bounds what windowed groups hold)."""
+        self.model = model
+        self.device = model.device
+        self.page_size = page_size
+        self.max_running = max_running
+        self.layout = CacheLayout.from_needs(model.cache_slots())
+        item = torch.empty((), dtype=model.dtype).element_size()
+        per_page = sum(self.layout.bytes_per_page(page_size, item))
+        max_pages = self._pages_that_fit(per_page, kv_mem_fraction, max_step_tokens or 8192)
+        if kv_pool_tokens is not None:
+            pages = kv_pool_tokens // page_size
+            if pages < 1:
+                raise ValueError(f"kv_pool_tokens={kv_pool_tokens} holds no page of {page_size} tokens")
+            if max_pages is not None and pages > max_pages:
+                raise ValueError(
+                    f"kv_pool_tokens={kv_pool_tokens} needs {pages} pages of {per_page} bytes; {max_pages} fit in memory"
+                )
+        else:
+            if max_pages is None or max_pages < 1:
+                raise RuntimeError("no memory left for the cache pool")
+            pages = max_pages
+        self.num_pages = pages
+        per_group = [pages for _ in self.layout.groups]
+        kw = {} if allocator_class is None else {"allocator_class": allocator_class}
+        self.cache = CacheManager(self.layout, page_size, per_group, max_running, max_step_tokens, **kw)
+        self.pool = KVPool(self.layout, page_size, per_group, max_running, model.dtype, self.device)
+        self.builder = BatchBuilder(self.device, len(self.layout.groups))
+        self.steps = 0
+
+    def _pages_that_fit(self, per_page: int, fraction: float, step_tokens: int) -> int | None:
+        if self.device.type != "cuda" or per_page == 0:
+            return None
+        free, _ = torch.cuda.mem_get_info(self.device)
+        spec = self.model.spec
+        widest = max([spec.hidden_size] + [b.feed_forward.spec.get("intermediate_size", 0) * 3 for b in self.model.blocks])
+        reserve = step_tokens * (spec.hidden_size * 8 + widest * 4 * 2) + self.max_running * spec.vocab_size * 8
+        return max(0, int((free - reserve) * fraction) // per_page)
+
+    # ------------------------------------------------------------------ request handles
+
+    def acquire(self) -> RequestCache:
+        return self.cache.acquire()
+
+    def release(self, rc: RequestCache) -> None:
+        self.cache.release(rc)
+
+    # ------------------------------------------------------------------ the step function
+
+    def step(self, rows: list[StepRow]) -> torch.Tensor | None:
+        """Run one batch. Each row's tokens continue its cache at position ``cache.num_tokens``.
+        Returns float32 logits ``[sum(len(row.want)), vocab]`` in row order (None if nothing is
+        wanted). Raises ``OutOfBlocks`` with every table unchanged if the pool cannot hold the step."""
+        if not rows:
+            return None
+        vocab = self.model.vocab_size
+        seen = set()
+        for r in rows:
+            if id(r.cache) in seen:
+                raise ValueError("a request appears twice in one step")
+            seen.add(id(r.cache))
+            if not r.tokens:
+                raise ValueError("a row without tokens")
+            if min(r.tokens) < 0 or max(r.tokens) >= vocab:
+                raise ValueError(f"token id out of range [0, {vocab})")
+            if r.want and not (0 <= min(r.want) and max(r.want) < len(r.tokens)):
+                raise ValueError("wanted place outside the row's tokens")
+        need = [0] * self.cache.num_groups
+        for r in rows:
+            for g, k in enumerate(self.cache.pages_needed(r.cache, len(r.tokens))):
+                need[g] += k
+        for g, (k, free) in enumerate(zip(need, self.cache.free_pages())):
+            if k > free:
+                raise OutOfBlocks(f"group {g}: the step needs {k} free pages, {free} free")
+        starts = [r.cache.num_tokens for r in rows]
+        for r in rows:
+            self.cache.extend(r.cache, len(r.tokens))
+        batch = self.builder.build(rows, starts)
+        logits = self.model.forward(batch, self.pool)
+        for r in rows:
+            self.cache.advance(r.cache)
+        self.steps += 1
+        return logits

@@ -1,0 +1,283 @@
+"""The kernel library as Python calls: every function checks shapes, dtypes and contiguity on the
+host, then launches hand-written HIP kernels on torch's current stream. There is no fallback:
+without a GPU or without the built library these calls raise.
+
+Tensors are torch tensors used as plain device buffers; no torch operator computes anything here.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import build
+
+_lib = None
+
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+_c_void, _c_int, _c_float, _c_ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+
+_ERRORS = {1: "bad argument", 2: "unsupported size", 3: "kernel launch failed"}
+
+_SIGNATURES = {
+    "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
+    "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
+    "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
+    "ms_qk_norm_rope_store": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int,
+                              _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
+                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
+}
+
+
+class KernelLibraryMissing(RuntimeError):
+    pass
+
+
+def library():
+    """The loaded kernel library; built first if no build of the current sources exists."""
+    global _lib
+    if _lib is None:
+        if not torch.cuda.is_available():
+            raise KernelLibraryMissing("no GPU is visible: the engine runs on HIP kernels only and has no CPU fallback")
+        try:
+            path = build.build_kernels()
+            lib = ctypes.CDLL(str(path))
+        except Exception as e:  # noqa: BLE001
+            raise KernelLibraryMissing(f"the HIP kernel library could not be built or loaded: {e}") from e
+        for name, args in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = _c_int
+        _lib = lib
+    return _lib
+
+
+def library_path() -> str:
+    return str(build.build_kernels())
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(code: int, what: str) -> None:
+    if code:
+        raise RuntimeError(f"{what}: {_ERRORS.get(code, code)}")
+
+
+def _dev(t: torch.Tensor, name: str, dtypes, ndim: int | None = None) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name} must be a tensor on the GPU")
+    if t.dtype not in (dtypes if isinstance(dtypes, tuple) else (dtypes,)):
+        raise TypeError(f"{name} has dtype {t.dtype}, expected {dtypes}")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} has {t.dim()} dimensions, expected {ndim}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _ptr(t) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------------------------- elementwise
+
+
+def embed(token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """``float32 [T, width]`` rows of ``table`` (float32 or bfloat16). Ids must be in range (the
+    caller checks them on the host before they are uploaded)."""
+    _dev(token_ids, "token_ids", I32, 1)
+    _dev(table, "table", (F32, BF16), 2)
+    out = torch.empty((token_ids.shape[0], table.shape[1]), dtype=F32, device=table.device)
+    _check(library().ms_embed(token_ids.data_ptr(), table.data_ptr(), int(table.dtype == BF16), out.data_ptr(),
+                              token_ids.shape[0], table.shape[1], _stream()), "embed")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None) -> torch.Tensor:
+    _dev(x, "x", F32, 2)
+    _dev(weight, "weight", (F32, BF16), 1)
+    if weight.shape[0] != x.shape[1]:
+        raise ValueError(f"norm weight has {weight.shape[0]} elements for width {x.shape[1]}")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    n = x.shape[0]
+    if rows is not None:
+        _dev(rows, "rows", I32, 1)
+        n = rows.shape[0]
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    _check(library().ms_rmsnorm(x.data_ptr(), weight.data_ptr(), int(weight.dtype == BF16), out.data_ptr(),
+                                int(out_dtype == BF16), _ptr(rows), n, x.shape[1], float(eps), _stream()), "rmsnorm")
+    return out
+
+
+def act_mul(gu: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """``act(gu[:, :I]) * gu[:, I:]`` for ``gu [T, 2 I]``."""
+    if activation != "silu":
+        raise NotImplementedError(f"activation {activation!r}")
+    _dev(gu, "gu", (F32, BF16), 2)
+    if gu.shape[1] % 2:
+        raise ValueError("gate/up buffer needs an even width")
+    inter = gu.shape[1] // 2
+    out = torch.empty((gu.shape[0], inter), dtype=gu.dtype, device=gu.device)
+    # grid.y carries the token index: split very long batches
+    for t0 in range(0, gu.shape[0], 32768):
+        n = min(32768, gu.shape[0] - t0)
+        _check(library().ms_silu_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, _stream()),
+               "silu_mul")
+    return out
+
+
+def cast(x: torch.Tensor, dtype) -> torch.Tensor:
+    if x.dtype == dtype:
+        return x
+    _dev(x, "x", (F32, BF16))
+    if dtype not in (F32, BF16):
+        raise TypeError(f"unsupported dtype {dtype}")
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _check(library().ms_cast(x.data_ptr(), int(x.dtype == BF16), out.data_ptr(), int(dtype == BF16), x.numel(), _stream()),
+           "cast")
+    return out
+
+
+# ------------------------------------------------------------------------------------- matrix products
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None) -> torch.Tensor:
+    """``x [M, K] @ weight [N, K]^T``. Either returns a new ``[M, N]`` tensor of ``out_dtype``, or adds
+    the product into the float32 tensor ``accumulate_into`` (the residual stream) and returns it.
+    The weight's dtype picks the arithmetic: float32 weights run the true 32-bit kernel (``x`` is
+    widened first if needed), bfloat16 weights the matrix-core kernel with float32 accumulation."""
+    _dev(x, "x", (F32, BF16), 2)
+    _dev(weight, "weight", (F32, BF16), 2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise ValueError(f"linear: x is [{m}, {k}], weight is {tuple(weight.shape)}")
+    if accumulate_into is not None:
+        _dev(accumulate_into, "accumulate_into", F32, 2)
+        if tuple(accumulate_into.shape) != (m, n):
+            raise ValueError(f"linear: accumulator is {tuple(accumulate_into.shape)}, expected {(m, n)}")
+        out = accumulate_into
+    else:
+        if out_dtype not in (F32, BF16):
+            raise TypeError(f"unsupported output dtype {out_dtype}")
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if weight.dtype == F32:
+        xa = cast(x, F32)
+        mode = 1 if accumulate_into is not None else (0 if out.dtype == F32 else 2)
+        _check(library().ms_gemm_f32(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
+               "gemm_f32")
+    else:
+        xa = cast(x, BF16)
+        mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
+        _check(library().ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
+               "gemm_bf16")
+    return out
+
+
+# ------------------------------------------------------------------------------------- attention
+
+
+def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq, rot_dim, k_cache, v_cache,
+                       num_heads, num_kv_heads, head_dim) -> None:
+    """In place on ``qkv [T, (Hq + 2 Hkv) D]``: per-head RMSNorm of q and k (if weights are given),
+    rotation by ``positions`` (if ``inv_freq`` is given), q written back, k and v stored into the
+    cache pages at ``slots`` (skipped when ``slots`` is None)."""
+    _dev(qkv, "qkv", (F32, BF16), 2)
+    t = qkv.shape[0]
+    if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {(num_heads + 2 * num_kv_heads) * head_dim}")
+    _dev(positions, "positions", I32, 1)
+    if positions.shape[0] != t:
+        raise ValueError("one position per token is needed")
+    if head_dim > 256 or head_dim < 1:
+        raise ValueError(f"head_dim {head_dim} is outside the kernels' range 1..256")
+    w_bf16 = 0
+    if q_weight is not None:
+        for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
+            _dev(w, nm, (F32, BF16), 1)
+            if w.shape[0] != head_dim:
+                raise ValueError(f"{nm} weight has {w.shape[0]} elements for head_dim {head_dim}")
+        if q_weight.dtype != k_weight.dtype:
+            raise TypeError("q_norm and k_norm weights differ in dtype")
+        w_bf16 = int(q_weight.dtype == BF16)
+    page_size = 1
+    if slots is not None:
+        _dev(slots, "slots", I32, 1)
+        if slots.shape[0] != t:
+            raise ValueError("one slot per token is needed")
+        for c, nm in ((k_cache, "k_cache"), (v_cache, "v_cache")):
+            _dev(c, nm, qkv.dtype, 4)
+            if c.shape[1] != num_kv_heads or c.shape[3] != head_dim:
+                raise ValueError(f"{nm} is {tuple(c.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
+        page_size = k_cache.shape[2]
+    if inv_freq is not None:
+        _dev(inv_freq, "inv_freq", F32, 1)
+        if rot_dim % 2 or rot_dim > head_dim or inv_freq.shape[0] != rot_dim // 2:
+            raise ValueError(f"rotation over {rot_dim} elements needs {rot_dim // 2} frequencies and head_dim >= it")
+    else:
+        rot_dim = 0
+    _check(library().ms_qk_norm_rope_store(
+        qkv.data_ptr(), int(qkv.dtype == BF16), positions.data_ptr(), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
+        float(eps), _ptr(inv_freq), int(rot_dim), _ptr(k_cache) if slots is not None else None,
+        _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, page_size, _stream()),
+        "qk_norm_rope_store")
+
+
+def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window):
+    """Attention of the batch's new tokens over the cache. ``qkv [T, >= Hq D]`` holds the queries
+    in its first ``Hq * D`` columns. Returns ``[T, Hq * D]``."""
+    _dev(qkv, "qkv", (F32, BF16), 2)
+    t = qkv.shape[0]
+    for c, nm in ((k_cache, "k_cache"), (v_cache, "v_cache")):
+        _dev(c, nm, qkv.dtype, 4)
+        if c.shape[1] != num_kv_heads or c.shape[3] != head_dim:
+            raise ValueError(f"{nm} is {tuple(c.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 up to 256")
+    if num_heads % num_kv_heads:
+        raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} KV heads")
+    if qkv.shape[1] < num_heads * head_dim:
+        raise ValueError("qkv is narrower than the query heads")
+    _dev(block_table, "block_table", I32, 2)
+    _dev(batch.token_row, "token_row", I32, 1)
+    _dev(batch.positions, "positions", I32, 1)
+    if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
+        raise ValueError("batch metadata does not match the number of tokens or rows")
+    out = torch.empty((t, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    _check(library().ms_paged_attention_generic(
+        qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16),
+        block_table.data_ptr(), block_table.shape[1], batch.token_row.data_ptr(), batch.positions.data_ptr(),
+        out.data_ptr(), t, num_heads, num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), _stream()),
+        "paged_attention")
+    return out
+
+
+# ------------------------------------------------------------------------------------- sampling
+
+
+def sample_rows(logits, temperature=None, top_p=None, seed=None, counter=None) -> torch.Tensor:
+    """``int32 [rows]`` token ids from float32 ``logits [rows, vocab]``. Without ``temperature`` every
+    row takes the first maximal index; with it, rows whose temperature is 0 still do."""
+    _dev(logits, "logits", F32, 2)
+    rows, vocab = logits.shape
+    if temperature is not None:
+        _dev(temperature, "temperature", F32, 1)
+        _dev(seed, "seed", I32, 1)
+        _dev(counter, "counter", I32, 1)
+        if top_p is not None:
+            _dev(top_p, "top_p", F32, 1)
+        for v in (temperature, seed, counter) + ((top_p,) if top_p is not None else ()):
+            if v.shape[0] != rows:
+                raise ValueError("one sampling parameter per row is needed")
+    out = torch.empty((rows,), dtype=I32, device=logits.device)
+    _check(library().ms_sample_rows(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
+                                    _ptr(counter), out.data_ptr(), _stream()), "sample_rows")
+    return out

@@ -1,0 +1,90 @@
+"""Grouped-query softmax attention over the paged cache.
+
+Per layer, in the reference's order (miniserve/model/qwen3.py:110-126): q/k/v projections without
+bias, per-head RMSNorm of q and k (one ``[head_dim]`` weight each, shared by all heads), rotation
+of q and k, store of k and v into the cache, causal attention in which query head ``h`` reads KV
+head ``h // (heads / kv_heads)`` with ``scale`` on the scores, output projection. Here the three
+projections are one matrix product over row-concatenated weights (as the reference's fused path
+does, miniserve/model/fused.py:204-206); norm, rotation and cache store are one kernel; the output
+projection adds into the residual stream in its epilogue.
+
+``window > 0`` restricts a query at position p to keys p-window+1 .. p (no counterpart in the
+reference). ``qk_norm_eps=None`` switches the per-head norms off; ``position`` may be ``none``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..config.spec import PartSpec
+from .base import KVNeed, Mixer, TensorSpec
+from .registry import part_class, register
+
+
+@register("mixer", "gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, spec: PartSpec, rt):
+        super().__init__(spec, rt)
+        self.prefix = spec.get("prefix", "")
+        self.hidden = int(spec["hidden_size"])
+        self.heads = int(spec["num_heads"])
+        self.kv_heads = int(spec["num_kv_heads"])
+        self.head_dim = int(spec["head_dim"])
+        self.scale = float(spec["scale"])
+        self.qk_norm_eps = spec.get("qk_norm_eps")
+        self.window = int(spec.get("window") or 0)
+        if self.heads % self.kv_heads:
+            raise ValueError(f"{self.heads} query heads are no multiple of {self.kv_heads} KV heads")
+        pos = spec.get("position") or PartSpec("none")
+        self.position = part_class("position", pos)(pos, rt)
+        self.qkv = self.o = self.q_norm = self.k_norm = None
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        p = spec.get("prefix", "")
+        h, d = int(spec["hidden_size"]), int(spec["head_dim"])
+        hq, hkv = int(spec["num_heads"]), int(spec["num_kv_heads"])
+        out = {
+            p + "q_proj.weight": TensorSpec((hq * d, h)),
+            p + "k_proj.weight": TensorSpec((hkv * d, h)),
+            p + "v_proj.weight": TensorSpec((hkv * d, h)),
+            p + "o_proj.weight": TensorSpec((h, hq * d)),
+        }
+        if spec.get("qk_norm_eps") is not None:
+            out[p + "q_norm.weight"] = TensorSpec((d,))
+            out[p + "k_norm.weight"] = TensorSpec((d,))
+        return out
+
+    def bind(self, tensors) -> None:
+        p = self.prefix
+        parts = [tensors[p + n + "_proj.weight"] for n in ("q", "k", "v")]
+        if len({t.dtype for t in parts}) != 1:
+            raise ValueError(f"{p}q/k/v projections are stored in different dtypes")
+        self.qkv = torch.cat(parts, dim=0).contiguous()
+        self.o = tensors[p + "o_proj.weight"]
+        if self.qk_norm_eps is not None:
+            self.q_norm = tensors[p + "q_norm.weight"]
+            self.k_norm = tensors[p + "k_norm.weight"]
+
+    def kv_need(self) -> KVNeed:
+        return KVNeed(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, batch, cache, state, residual) -> None:
+        ops = self.rt.ops
+        qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype)
+        rot = self.position.rotation()
+        ops.qk_norm_rope_store(
+            qkv, batch.positions, cache.slots if cache.writes else None,
+            self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps),
+            rot.inv_freq if rot is not None else None, rot.dim if rot is not None else 0,
+            cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
+        )
+        out = ops.paged_attention(
+            qkv, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
+            self.scale, self.window,
+        )
+        ops.linear(out, self.o, accumulate_into=residual)
+
+    def parameters_bytes(self) -> int:
+        ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else [])
+        return sum(t.numel() * t.element_size() for t in ts)

@@ -1,0 +1,142 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part is built from a ``PartSpec`` (its sizes and constants) and a ``Runtime`` (compute dtype,
+device, kernels); it declares the tensors it needs under its own prefix and receives exactly
+those. No part knows which model it is in. The kinds:
+
+* ``Norm``            ``forward(x_f32, rows=None) -> y``            (residual stream in, compute dtype out)
+* ``PositionEncoding`` ``rotation() -> Rotation | None``            (what a mixer's q/k are turned by)
+* ``Mixer``           ``forward(x, batch, cache, state, residual)`` (adds its output to ``residual``)
+* ``FeedForward``     ``forward(x, residual)``                      (adds its output to ``residual``)
+* ``Block``           ``forward(residual, batch, cache, state)``    (where norms and sums sit)
+* ``Embedding``       ``forward(token_ids) -> residual``            (float32 ``[T, width]``)
+* ``Head``            ``forward(x) -> logits``                      (float32 ``[rows, vocab]``)
+
+The residual stream is float32 in every compute dtype: sums of layer outputs are never rounded
+to bfloat16. Mixers and feed-forwards add into it (so a matrix product can do the sum in its
+epilogue) instead of returning a tensor.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import TYPE_CHECKING, Any, Mapping
+
+from ..config.spec import PartSpec
+
+if TYPE_CHECKING:  # pragma: no cover
+    import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part expects in the checkpoint. ``kind``: ``"float"`` tensors follow the compute
+    dtype (a tensor stored in 32-bit stays 32-bit); ``"int"`` tables are kept as int32."""
+
+    shape: tuple[int, ...]
+    kind: str = "float"
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values a mixer keeps per token: ``window == 0`` keeps all of them, ``window > 0``
+    only the last ``window`` (older pages may be given back)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size a mixer keeps (shape per request, torch dtype name)."""
+
+    shape: tuple[int, ...]
+    dtype: str = "float32"
+
+
+@dataclass(frozen=True)
+class Rotation:
+    """Rotary position encoding as a mixer's kernels need it: the first ``dim`` elements of each
+    head are turned in pairs (j, j + dim/2) by ``position * inv_freq[j]``."""
+
+    dim: int
+    inv_freq: Any  # float32 device tensor [dim / 2]
+
+
+class Runtime:
+    """What every part is built with: the compute dtype, the device and the kernel library."""
+
+    def __init__(self, dtype, device, ops):
+        self.dtype = dtype  # torch.float32 or torch.bfloat16
+        self.device = device
+        self.ops = ops
+
+
+class Part:
+    """Base of all parts. Subclasses override ``tensors`` (static: needs no device) and ``bind``."""
+
+    kind: str = ""
+
+    def __init__(self, spec: PartSpec, rt: Runtime | None):
+        self.spec = spec
+        self.rt = rt
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        """Checkpoint tensors of this part, named relative to the layer prefix (or absolutely
+        for parts outside layers)."""
+        return {}
+
+    def bind(self, tensors: Mapping[str, "torch.Tensor"]) -> None:
+        """Receive the tensors declared by ``tensors`` (same names), already on the device."""
+
+    def parameters_bytes(self) -> int:
+        """Bytes of weights a decode step reads from this part (for the bandwidth model)."""
+        return 0
+
+
+class Norm(Part):
+    def forward(self, x, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotation(self) -> Rotation | None:
+        return None
+
+
+class Mixer(Part):
+    def kv_need(self) -> KVNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x, batch, cache, state, residual) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, residual) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    def __init__(self, spec: PartSpec, rt, mixer: Mixer, feed_forward: FeedForward):
+        super().__init__(spec, rt)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+
+    def forward(self, residual, batch, cache, state) -> None:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, token_ids):
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, x):
+        raise NotImplementedError

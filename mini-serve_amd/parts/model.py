@@ -1,0 +1,114 @@
+"""The generic decoder: parts assembled from a ``ModelSpec`` and run in the order it lists.
+
+One class serves every registered architecture; an architecture is its typed configuration's
+``to_spec``. The model owns no cache: the step function hands it a batch and the pool's views.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+from ..config.spec import ModelSpec
+from .base import KVNeed, Runtime, StateNeed, TensorSpec
+from .registry import part_class
+
+
+def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
+    """Every checkpoint tensor of the model with its shape, collected from the parts' own
+    declarations (the reference lists them in one flat function, miniserve/model/weights.py:60-91)."""
+    out: dict[str, TensorSpec] = {}
+
+    def add(tensors: dict[str, TensorSpec], prefix: str = "") -> None:
+        for name, ts in tensors.items():
+            full = prefix + name
+            if full in out and out[full] != ts:
+                raise ValueError(f"tensor {full} is declared twice with different shapes")
+            out[full] = ts
+
+    add(part_class("embedding", spec.embedding).tensors(spec.embedding))
+    for layer in spec.layers:
+        add(part_class("block", layer.block).tensors(layer.block), layer.prefix)
+        add(part_class("mixer", layer.mixer).tensors(layer.mixer), layer.prefix)
+        add(part_class("feed_forward", layer.feed_forward).tensors(layer.feed_forward), layer.prefix)
+    add(part_class("norm", spec.final_norm).tensors(spec.final_norm))
+    add(part_class("head", spec.head).tensors(spec.head))
+    return out
+
+
+@dataclass(frozen=True)
+class CacheSlotNeed:
+    """What one cache slot of the run order holds: paged keys/values and/or fixed-size state."""
+
+    slot: int
+    kv: KVNeed | None
+    state: StateNeed | None
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, weights: dict, rt: Runtime):
+        self.spec = spec
+        self.rt = rt
+        self.dtype = rt.dtype
+        self.device = rt.device
+        self.vocab_size = spec.vocab_size
+
+        def local(prefix: str, names) -> dict:
+            return {n: weights[prefix + n] for n in names}
+
+        self.embedding = part_class("embedding", spec.embedding)(spec.embedding, rt)
+        self.embedding.bind(weights)
+        self.blocks = []
+        for layer in spec.layers:
+            mixer = part_class("mixer", layer.mixer)(layer.mixer, rt)
+            mixer.bind(local(layer.prefix, type(mixer).tensors(layer.mixer)))
+            ffn = part_class("feed_forward", layer.feed_forward)(layer.feed_forward, rt)
+            ffn.bind(local(layer.prefix, type(ffn).tensors(layer.feed_forward)))
+            block = part_class("block", layer.block)(layer.block, rt, mixer, ffn)
+            block.bind(local(layer.prefix, type(block).tensors(layer.block)))
+            self.blocks.append(block)
+        self.final_norm = part_class("norm", spec.final_norm)(spec.final_norm, rt)
+        self.final_norm.bind(weights)
+        self.head = part_class("head", spec.head)(spec.head, rt)
+        self.head.bind(weights)
+
+    # ------------------------------------------------------------------ cache needs
+
+    def cache_slots(self) -> list[CacheSlotNeed]:
+        """One entry per cache slot of the run order, from the mixer that writes it."""
+        needs: dict[int, CacheSlotNeed] = {}
+        for e in self.spec.run_order:
+            if e.cache is None:
+                continue
+            mixer = self.blocks[e.layer].mixer
+            need = CacheSlotNeed(e.cache, mixer.kv_need(), mixer.state_need())
+            if e.writes_cache:
+                needs[e.cache] = need
+            elif (needs[e.cache].kv, needs[e.cache].state) != (need.kv, need.state):
+                raise ValueError(
+                    f"layer {e.layer} reads cache slot {e.cache} but needs {need}, the slot holds {needs[e.cache]}"
+                )
+        return [needs[s] for s in sorted(needs)]
+
+    # ------------------------------------------------------------------ forward
+
+    def forward(self, batch, pool):
+        """Run the batch's tokens through every run-order entry and return float32 logits
+        ``[len(batch.want_rows), vocab]`` at the wanted flat token indices."""
+        residual = self.embedding.forward(batch.token_ids)
+        for e in self.spec.run_order:
+            cache = pool.view(e.cache, batch, e.writes_cache) if e.cache is not None else None
+            state = pool.state_view(e.cache, batch) if e.cache is not None else None
+            self.blocks[e.layer].forward(residual, batch, cache, state)
+        if batch.num_wanted == 0:
+            return None
+        x = self.final_norm.forward(residual, rows=batch.want_rows)
+        return self.head.forward(x)
+
+    def decode_read_bytes(self) -> int:
+        """Bytes of weights one decode step reads: every run-order entry's layer once, the final
+        norm and the head (embedding rows are only gathered)."""
+        total = self.final_norm.parameters_bytes() + self.head.parameters_bytes()
+        for e in self.spec.run_order:
+            b = self.blocks[e.layer]
+            total += b.parameters_bytes() + b.mixer.parameters_bytes() + b.feed_forward.parameters_bytes()
+        return total

@@ -1,0 +1,309 @@
+"""Each HIP kernel alone against a plain float32/float64 torch expression of the same op, at sizes
+other than the engine's test models: widths and vocabularies that are no power of two, head sizes
+in steps of 16, odd head counts and groups, rows that do not fill a tile."""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from miniserve_amd.kernels import ops as o
+
+    o.library()
+    return o
+
+
+def rand(shape, dtype=F32, seed=0, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, rel, what=""):
+    got, want = got.double().cpu(), want.double().cpu()
+    scale = float(want.abs().max()) or 1.0
+    err = float((got - want).abs().max())
+    assert err <= rel * scale, f"{what}: max |diff| {err:.3e} > {rel * scale:.3e}"
+
+
+# ------------------------------------------------------------------------------------------ elementwise
+
+
+@pytest.mark.parametrize("table_dtype", [F32, BF16])
+def test_embed(ops, table_dtype):
+    table = rand((379, 96), table_dtype, 1)
+    ids = torch.tensor([0, 378, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = ops.embed(ids, table)
+    assert out.dtype == F32
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("width", [96, 1000, 5120])
+@pytest.mark.parametrize("w_dtype,out_dtype", [(F32, F32), (BF16, BF16), (F32, BF16), (BF16, F32)])
+def test_rmsnorm(ops, width, w_dtype, out_dtype):
+    x = rand((7, width), F32, 2, 3.0)
+    w = rand((width,), w_dtype, 3)
+    eps = 1e-5
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps) * w.double()
+    got = ops.rmsnorm(x, w, eps, out_dtype)
+    close(got, want, 1e-6 if out_dtype == F32 else 5e-3, "rmsnorm")
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    got = ops.rmsnorm(x, w, eps, out_dtype, rows)
+    close(got, want[rows.long()], 1e-6 if out_dtype == F32 else 5e-3, "rmsnorm rows")
+
+
+def test_rmsnorm_eps_enters(ops):
+    x = rand((2, 64), F32, 4, 1e-3)
+    w = torch.ones(64, device=DEV)
+    a, b = ops.rmsnorm(x, w, 1e-6, F32), ops.rmsnorm(x, w, 1e-5, F32)
+    assert (a - b).abs().max() > 1e-2  # at this scale eps is of the size of mean(x^2)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_silu_mul(ops, dtype):
+    gu = rand((5, 2 * 224), dtype, 5, 2.0)
+    g, u = gu[:, :224].double(), gu[:, 224:].double()
+    want = g / (1 + torch.exp(-g)) * u
+    close(ops.act_mul(gu), want, 1e-6 if dtype == F32 else 5e-3, "silu_mul")
+    z = torch.zeros((1, 8), dtype=dtype, device=DEV)
+    assert float(ops.act_mul(z).abs().max()) == 0.0
+
+
+# ------------------------------------------------------------------------------------------ matrix products
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 379, 96), (130, 200, 224), (64, 70, 37), (3, 1024, 3072)])
+def test_gemm_f32(ops, m, n, k):
+    x, w = rand((m, k), F32, 6), rand((n, k), F32, 7)
+    want = x.double() @ w.double().T
+    close(ops.linear(x, w, out_dtype=F32), want, 2e-6, "gemm f32")
+    acc = rand((m, n), F32, 8)
+    before = acc.clone()
+    ops.linear(x, w, accumulate_into=acc)
+    close(acc, before.double() + want, 2e-6, "gemm f32 accumulate")
+    close(ops.linear(x, w, out_dtype=BF16), want, 5e-3, "gemm f32 -> bf16")
+
+
+def test_gemm_f32_rows_do_not_depend_on_batch(ops):
+    x, w = rand((130, 224), F32, 9), rand((379, 224), F32, 10)
+    whole = ops.linear(x, w, out_dtype=F32)
+    for lo, hi in ((0, 1), (63, 66), (100, 130)):
+        assert torch.equal(ops.linear(x[lo:hi].contiguous(), w, out_dtype=F32), whole[lo:hi])
+
+
+@pytest.mark.parametrize("m", [1, 7, 16, 17, 33, 64, 65, 200, 1000])
+@pytest.mark.parametrize("n,k", [(379, 96), (192, 224), (1024, 1024), (100, 100), (4096, 128)])
+def test_gemm_bf16(ops, m, n, k):
+    x, w = rand((m, k), BF16, 11), rand((n, k), BF16, 12)
+    want = x.double() @ w.double().T
+    close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
+    close(ops.linear(x, w, out_dtype=BF16), want, 5e-3, "gemm bf16 -> bf16")
+    acc = rand((m, n), F32, 13)
+    before = acc.clone()
+    ops.linear(x, w, accumulate_into=acc)
+    close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
+
+
+def test_linear_with_float32_weights_in_bfloat16_mode(ops):
+    x, w = rand((9, 96), BF16, 14), rand((50, 96), F32, 15)
+    close(ops.linear(x, w, out_dtype=BF16), x.double() @ w.double().T, 5e-3, "f32 weights, bf16 activations")
+
+
+# ------------------------------------------------------------------------------------------ attention pieces
+
+
+def plain_rope(x, pos, inv_freq, rot):
+    """x [T, heads, D] float64; pairs (j, j + rot/2) of the first rot elements."""
+    ang = pos.float()[:, None] * inv_freq[None, :]  # float32 as the engine forms it
+    ang = ang.double()
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    half = rot // 2
+    a, b = x[..., :half], x[..., half:rot]
+    out = x.clone()
+    out[..., :half] = a * cos - b * sin
+    out[..., half:rot] = b * cos + a * sin
+    return out
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 1, 32, 32, 16), (3, 3, 48, 24, 8), (5, 5, 256, 256, 4), (16, 8, 128, 128, 16)])
+def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
+    t, pages, eps = 11, 9, 1e-5
+    qkv = rand((t, (hq + 2 * hkv) * d), dtype, 16)
+    qw, kw = rand((d,), dtype, 17) + 1, rand((d,), dtype, 18) + 1
+    pos = torch.tensor([0, 1, 2, 3, 40, 41, 700, 5, 6, 7, 4000], dtype=torch.int32, device=DEV)
+    perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(1))[:t]
+    slots = perm.to(torch.int32).to(DEV)
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    kc = torch.full((pages, hkv, page, d), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, hkv, page, d), 7.0, dtype=dtype, device=DEV)
+    ref = qkv.double().view(t, hq + 2 * hkv, d)
+    q, k, v = ref[:, :hq], ref[:, hq : hq + hkv], ref[:, hq + hkv :]
+
+    def norm(x, w):
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
+
+    qn = plain_rope(norm(q, qw), pos, inv_freq, rot)
+    kn = plain_rope(norm(k, kw), pos, inv_freq, rot)
+    work = qkv.clone()
+    ops.qk_norm_rope_store(work, pos, slots, qw, kw, eps, inv_freq, rot, kc, vc, hq, hkv, d)
+    tol = 2e-6 if dtype == F32 else 5e-3
+    close(work.view(t, hq + 2 * hkv, d)[:, :hq], qn, tol, "q")
+    sl = slots.long()
+    got_k = kc.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)
+    got_v = vc.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)
+    close(got_k[sl], kn, tol, "k in cache")
+    assert torch.equal(got_v[sl].double(), v), "v is stored as it is"
+    untouched = torch.ones(pages * page, dtype=torch.bool)
+    untouched[sl.cpu()] = False
+    assert float((got_k[untouched.to(DEV)] - 7).abs().max()) == 0 and float((got_v[untouched.to(DEV)] - 7).abs().max()) == 0
+    # position 0 is the identity of the rotation
+    close(work.view(t, hq + 2 * hkv, d)[0, :hq], norm(q, qw)[0], tol, "position 0")
+
+
+class _Batch:
+    pass
+
+
+def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=0):
+    """Rows with ``starts[i]`` cached tokens and ``lens_new[i]`` new ones; scattered pages."""
+    g = torch.Generator().manual_seed(seed)
+    b = len(lens_new)
+    totals = [s + n for s, n in zip(starts, lens_new)]
+    blocks = [-(-tt // page) for tt in totals]
+    pages = sum(blocks) + 3
+    order = torch.randperm(pages, generator=g).tolist()
+    width = max(blocks)
+    table = torch.full((b, width), -1, dtype=torch.int32)
+    kc = rand((pages, hkv, page, d), dtype, seed + 1)
+    vc = rand((pages, hkv, page, d), dtype, seed + 2)
+    at = 0
+    for i, nb in enumerate(blocks):
+        table[i, :nb] = torch.tensor(order[at : at + nb], dtype=torch.int32)
+        at += nb
+    t = sum(lens_new)
+    q = rand((t, (hq + 2 * hkv) * d), dtype, seed + 3)
+    batch = _Batch()
+    batch.num_rows = b
+    batch.token_row = torch.tensor([i for i, n in enumerate(lens_new) for _ in range(n)], dtype=torch.int32, device=DEV)
+    batch.positions = torch.tensor([s + j for s, n in zip(starts, lens_new) for j in range(n)], dtype=torch.int32, device=DEV)
+    scale = d**-0.5
+    got = ops.paged_attention(q, kc, vc, table.to(DEV), batch, hq, hkv, d, scale, window)
+    want = torch.empty((t, hq, d), dtype=torch.float64)
+    qd = q.double().cpu().view(t, hq + 2 * hkv, d)[:, :hq]
+    kcd, vcd = kc.double().cpu(), vc.double().cpu()
+    tok = 0
+    for i in range(b):
+        keys = torch.stack([kcd[table[i, p // page], :, p % page] for p in range(totals[i])])  # [len, hkv, d]
+        vals = torch.stack([vcd[table[i, p // page], :, p % page] for p in range(totals[i])])
+        for j in range(lens_new[i]):
+            p = starts[i] + j
+            lo = max(0, p - window + 1) if window else 0
+            for h in range(hq):
+                kh = h // (hq // hkv)
+                s = (keys[lo : p + 1, kh] @ qd[tok, h]) * scale
+                w = torch.softmax(s, 0)
+                want[tok, h] = w @ vals[lo : p + 1, kh]
+            tok += 1
+    close(got.view(t, hq, d), want, 2e-6 if dtype == F32 else 8e-3, f"attention {hq}/{hkv}/{d} window {window}")
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize(
+    "hq,hkv,d,page,lens_new,starts,window",
+    [
+        (4, 2, 16, 16, [5, 1, 40], [0, 17, 3], 0),
+        (6, 1, 32, 16, [1, 1, 1, 1], [0, 15, 16, 130], 0),
+        (3, 3, 48, 8, [70, 2], [0, 100], 24),
+        (16, 8, 128, 16, [33, 1], [31, 200], 0),
+        (5, 5, 256, 4, [3, 9], [64, 0], 7),
+        (8, 2, 64, 16, [130], [0], 0),
+    ],
+)
+def test_paged_attention(ops, dtype, hq, hkv, d, page, lens_new, starts, window):
+    attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window)
+
+
+def test_attention_one_token_returns_its_value(ops):
+    """A sequence of one token: softmax over one key is 1, so the output is v."""
+    hq, hkv, d, page = 4, 2, 32, 16
+    q = rand((1, (hq + 2 * hkv) * d), F32, 20)
+    kc, vc = rand((2, hkv, page, d), F32, 21), rand((2, hkv, page, d), F32, 22)
+    batch = _Batch()
+    batch.num_rows = 1
+    batch.token_row = torch.zeros(1, dtype=torch.int32, device=DEV)
+    batch.positions = torch.zeros(1, dtype=torch.int32, device=DEV)
+    table = torch.tensor([[1]], dtype=torch.int32, device=DEV)
+    out = ops.paged_attention(q, kc, vc, table, batch, hq, hkv, d, d**-0.5, 0).view(hq, d)
+    for h in range(hq):
+        assert torch.equal(out[h], vc[1, h // 2, 0])
+
+
+def test_attention_refuses_unsupported_head_size(ops):
+    q = rand((1, 3 * 24), F32, 23)
+    kc = rand((1, 1, 16, 24), F32, 24)
+    batch = _Batch()
+    batch.num_rows = 1
+    batch.token_row = torch.zeros(1, dtype=torch.int32, device=DEV)
+    batch.positions = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="head_dim 24"):
+        ops.paged_attention(q, kc, kc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), batch, 1, 1, 24, 1.0, 0)
+
+
+# ------------------------------------------------------------------------------------------ sampling
+
+
+def test_argmax_takes_the_first_maximum(ops):
+    logits = rand((4, 379), F32, 25)
+    logits[0, [3, 7]] = 50.0
+    logits[3, [30, 5]] = 60.0
+    out = ops.sample_rows(logits).cpu().tolist()
+    assert out[0] == 3 and out[3] == 5
+    assert out[1] == int(logits[1].argmax()) and out[2] == int(logits[2].argmax())
+
+
+def _as_i32(values):
+    return torch.tensor([v - (1 << 32) if v >= (1 << 31) else v for v in values], dtype=torch.int32, device=DEV)
+
+
+@pytest.mark.parametrize("top_p", [1.0, 0.9, 0.3])
+def test_sampling_matches_plain(ops, top_p):
+    from plain import qwen3_plain as P
+
+    vocab, rows = 517, 12
+    logits = rand((rows, vocab), F32, 26, 3.0)
+    temps = [0.0, 0.8, 1.0, 2.0] * 3
+    seeds = [1, 2**32 - 1, 12345, 99, 7, 2**31, 0, 5, 6, 7, 8, 9]
+    counters = [0, 5, 17, 300, 1, 2, 3, 4, 40, 41, 42, 43]
+    got = ops.sample_rows(
+        logits, torch.tensor(temps, device=DEV), torch.full((rows,), top_p, device=DEV), _as_i32(seeds),
+        torch.tensor(counters, dtype=torch.int32, device=DEV),
+    ).cpu().tolist()
+    host = logits.cpu().numpy()
+    want = [P.sample(host[i], temps[i], seeds[i], counters[i], top_p) for i in range(rows)]
+    assert got == want
+
+
+def test_sampling_frequencies_follow_softmax(ops):
+    base = torch.tensor([2, 1, 0.5, 0, -1, -3, 1.5, 0.2], device=DEV)
+    n = 50000
+    logits = base.repeat(n, 1).contiguous()
+    for temp in (0.5, 1.0, 2.0):
+        toks = ops.sample_rows(
+            logits, torch.full((n,), temp, device=DEV), None, torch.arange(n, dtype=torch.int32, device=DEV),
+            torch.zeros(n, dtype=torch.int32, device=DEV),
+        )
+        freq = torch.bincount(toks.long(), minlength=8).double().cpu() / n
+        want = torch.softmax(base.double().cpu() / temp, 0)
+        assert float((freq - want).abs().max()) < 0.01
