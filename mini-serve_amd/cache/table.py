@@ -71,6 +71,10 @@ class BlockTable:
             raise IndexError(f"position {start} lies in a page that was given back")
         return [self.blocks[p // bs] * bs + p % bs for p in range(start, self.num_tokens)]
 
+    def tail_slots_into(self, n: int, out) -> None:
+        """``tail_slots(n)`` written into the int32 array ``out`` (its first ``n`` entries)."""
+        out[:n] = self.tail_slots(n)
+
     def rewind(self, n: int) -> None:
         if not 0 <= n <= self.num_tokens:
             raise IndexError(f"cannot rewind {n} of {self.num_tokens} tokens")
@@ -106,6 +110,12 @@ def pack_tables(tables, out, pad_rows: int = 0, pad_block: int = 0) -> int:
     rows = len(tables) + pad_rows
     if pad_rows < 0:
         raise ValueError("pad_rows must be >= 0")
+    if tables and not isinstance(tables[0], BlockTable):
+        from .native import pack_native
+
+        if out.ndim != 2 or not out.flags.c_contiguous:
+            raise ValueError("packing buffer must be a contiguous matrix")
+        return pack_native(tables, out, pad_rows, pad_block)
     if out.ndim != 2 or out.shape[0] < rows:
         raise ValueError(f"packing buffer too small: need {rows} rows, got {out.shape}")
     width = out.shape[1]

@@ -67,7 +67,7 @@ class BatchBuilder:
         lens = [len(r.tokens) for r in rows]
         T = sum(lens)
         n_want = sum(len(r.want) for r in rows)
-        widths = [max(1, max(len(r.cache.tables[g].blocks) for r in rows)) for g in range(self.num_groups)]
+        widths = [max(1, max(r.cache.tables[g].num_blocks for r in rows)) for g in range(self.num_groups)]
 
         seg = {}
         off = 0
@@ -113,7 +113,7 @@ class BatchBuilder:
             sl = view(f"slots{g}")
             t = 0
             for r, n in zip(rows, lens):
-                sl[t : t + n] = r.cache.tables[g].tail_slots(n)
+                r.cache.tables[g].tail_slots_into(n, sl[t : t + n])
                 t += n
             pack_tables([r.cache.tables[g] for r in rows], view(f"table{g}").reshape(B, widths[g]))
 

@@ -30,6 +30,8 @@ class ModelRunner:
         max_running: int = 64,
         max_step_tokens: int | None = None,
         allocator_class=None,
+        decode_graph: bool = False,
+        decode_graph_max_bs: int | None = None,
     ):
         """``kv_pool_tokens``: exact pool size in tokens (rounded down to whole pages; an error if
         it holds no page or does not fit, never clipped; miniserve/engine/model_runner.py:99-108);

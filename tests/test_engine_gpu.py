@@ -1,0 +1,167 @@
+"""Generation through the Python entry point and the command line against the plain
+implementation: greedy tokens, long decoding, chunked and unchunked prefill, a pool so small that
+requests are preempted and recomputed, sampled requests beside greedy ones."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from models import TINY, make_folder
+from plain import qwen3_plain as P
+from plain.model_folder import read_model_folder
+from replay_util import ROOT
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_folder(root, name) for name in TINY}
+
+
+def engine(folder, dtype="float32", **kw):
+    from miniserve_amd.engine.engine import Engine
+    from miniserve_amd.loading import load_model
+
+    return Engine(load_model(folder, dtype, "cuda:0"), **kw)
+
+
+def prompts_for(cfg, lens, seed=3):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in lens]
+
+
+@pytest.mark.parametrize("name", sorted(TINY))
+@pytest.mark.parametrize("chunk", [0, 16, 2048])
+def test_greedy_generation_equals_plain(name, chunk, folders):
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders[name])
+    prompts = prompts_for(cfg, [1, 9, 40, 17])
+    want = [P.greedy(cfg, w, p, 16) for p in prompts]
+    eng = engine(folders[name], kv_pool_tokens=512, max_running=4, chunked_prefill_size=chunk)
+    got = eng.generate(prompts, SamplingParams(max_new_tokens=16))
+    assert got == want
+    assert eng.runner.cache.idle
+
+
+def test_preemption_and_recompute_change_nothing(folders):
+    """A pool that cannot hold all requests at once: some are preempted, prefilled again with
+    their output kept, and still produce the tokens they produce alone."""
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyB"])
+    prompts = prompts_for(cfg, [30, 45, 20, 38, 25, 41], seed=4)
+    want = [P.greedy(cfg, w, p, 24) for p in prompts]
+    eng = engine(folders["tinyB"], kv_pool_tokens=16 * 12, max_running=6, chunked_prefill_size=32)
+    got = eng.generate(prompts, SamplingParams(max_new_tokens=24))
+    assert eng.scheduler.num_preemptions > 0, "the pool was meant to be too small"
+    assert got == want
+    assert eng.runner.cache.idle
+
+
+def test_long_decoding(folders):
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyA"])
+    prompt = prompts_for(cfg, [3], seed=5)[0]
+    want = P.greedy(cfg, w, prompt, 120)
+    eng = engine(folders["tinyA"], kv_pool_tokens=256)
+    assert eng.generate([prompt], SamplingParams(max_new_tokens=120)) == [want]
+
+
+def test_stop_token_is_kept(folders):
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyA"])
+    prompt = prompts_for(cfg, [12], seed=6)[0]
+    free = P.greedy(cfg, w, prompt, 10)
+    stop = free[4]
+    cut = free[: free.index(stop) + 1]
+    eng = engine(folders["tinyA"], kv_pool_tokens=256)
+    assert eng.generate([prompt], SamplingParams(max_new_tokens=10, stop_token_ids=frozenset({stop}))) == [cut]
+
+
+def test_sampled_requests_reproduce_beside_greedy_ones(folders):
+    """Temperature sampling with a request seed: the same tokens alone, in a batch, and after
+    preemption; equal to the plain sampler run on the plain logits."""
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyB"])
+    prompts = prompts_for(cfg, [14, 33, 21, 8], seed=7)
+    params = [SamplingParams(12, temperature=t, top_p=tp, seed=s) for t, tp, s in
+              ((0.8, 1.0, 11), (0.0, 1.0, None), (0.8, 0.9, 2**32 - 1), (1.5, 1.0, 0))]
+
+    def plain_run(p, sp):
+        ids, out = list(p), []
+        for _ in range(sp.max_new_tokens):
+            tok = P.sample(P.logits(cfg, w, ids)[-1], sp.temperature, sp.seed or 0, len(ids), sp.top_p)
+            out.append(tok)
+            ids.append(tok)
+        return out
+
+    want = [plain_run(p, sp) for p, sp in zip(prompts, params)]
+    for pool in (1024, 16 * 7):
+        eng = engine(folders["tinyB"], kv_pool_tokens=pool, max_running=4, chunked_prefill_size=16)
+        reqs = [eng.add_request(p, sp) for p, sp in zip(prompts, params)]
+        while eng.has_unfinished:
+            eng.step()
+        assert [r.output_ids for r in reqs] == want
+
+
+def test_abort_gives_pages_back(folders):
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, _ = read_model_folder(folders["tinyA"])
+    eng = engine(folders["tinyA"], kv_pool_tokens=512, max_running=4)
+    reqs = [eng.add_request(p, SamplingParams(50)) for p in prompts_for(cfg, [20, 30], seed=8)]
+    for _ in range(5):
+        eng.step()
+    eng.abort(reqs[0].rid)
+    eng.abort(reqs[0].rid)  # idempotent
+    while eng.has_unfinished:
+        eng.step()
+    assert len(reqs[1].output_ids) == 50 and len(reqs[0].output_ids) < 50
+    assert eng.runner.cache.idle
+
+
+def test_bfloat16_tokens_stay_near_the_best(folders):
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyB"])
+    prompts = prompts_for(cfg, [25, 60], seed=9)
+    eng = engine(folders["tinyB"], dtype="bfloat16", kv_pool_tokens=512)
+    for p, out in zip(prompts, eng.generate(prompts, SamplingParams(16))):
+        for i, tok in enumerate(out):
+            row = P.logits(cfg, w, p + out[:i])[-1]
+            assert row.max() - row[tok] <= 0.05 * np.abs(row).max()
+
+
+def test_command_line_generate(folders):
+    cfg, w = read_model_folder(folders["tinyA"])
+    prompt = prompts_for(cfg, [6], seed=10)[0]
+    res = subprocess.run(
+        [sys.executable, "-m", "miniserve_amd", "generate", "--model", str(folders["tinyA"]), "--dtype", "float32",
+         "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "8", "--kv-pool-tokens", "256"],
+        capture_output=True, text=True, cwd=str(ROOT), timeout=110,
+    )
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert json.loads(res.stdout.strip().splitlines()[-1])["outputs"] == [P.greedy(cfg, w, prompt, 8)]
+
+
+def test_stress_run_finishes_and_returns_every_page(folders):
+    res = subprocess.run(
+        [sys.executable, "-m", "miniserve_amd", "stress", "--model", str(folders["tinyB"]), "--num-requests", "24",
+         "--prompt-len", "4", "90", "--max-new-tokens", "1", "30", "--kv-pool-tokens", "640", "--max-running", "8",
+         "--chunked-prefill-size", "64", "--temperature", "0.7", "--top-p", "0.9"],
+        capture_output=True, text=True, cwd=str(ROOT), timeout=110,
+    )
+    assert res.returncode == 0, res.stdout[-1000:] + res.stderr[-2000:]
+    report = json.loads(res.stdout.strip().splitlines()[-1])
+    assert report["finished"] == 24 and report["idle"]
