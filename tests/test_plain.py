@@ -1,0 +1,235 @@
+"""Pins of the plain implementation beside the reference's text: special cases that reduce to a
+library routine, and invariants, each chosen so that a plausible mistake fails it (a wrong sign or
+pairing in the rotation, a norm in the wrong place or with the wrong eps, a mask off by one, a wrong
+head-to-group map). The reference's own numeric tests compare with a library model on downloaded
+weights (tests/test_consistency.py:68-145) and hold no vectors that could be reused here."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from models import TINY
+from miniserve_amd.weights.random_init import write_model_folder
+from plain import qwen3_plain as P
+from plain.model_folder import read_model_folder
+
+rng = np.random.default_rng(0)
+
+
+# ------------------------------------------------------------------------------------------ norm
+
+
+def test_rms_norm_formula_and_eps():
+    x = rng.standard_normal((5, 12)) * 3
+    w = rng.uniform(0.5, 1.5, 12)
+    eps = 1e-5
+    want = x / np.sqrt((x**2).mean(-1, keepdims=True) + eps) * w
+    assert np.allclose(P.rms_norm(x, w, eps), want, rtol=1e-14)
+    ones = np.ones(12)
+    y = P.rms_norm(x, ones, eps)
+    ms = (x**2).mean(-1)
+    assert np.allclose((y**2).mean(-1), ms / (ms + eps), rtol=1e-12)  # the weight is plain, not 1 + w
+    assert np.allclose(P.rms_norm(7 * x, ones, 0.0), P.rms_norm(x, ones, 0.0), rtol=1e-12)  # scale-free as eps -> 0
+    small = x * 1e-3
+    assert np.abs(P.rms_norm(small, ones, 1e-6) - P.rms_norm(small, ones, 1e-5)).max() > 1e-2  # eps really enters
+    assert not np.allclose(P.rms_norm(x, w, eps), x - x.mean(-1, keepdims=True))  # no mean is removed
+
+
+# ------------------------------------------------------------------------------------------ rotation
+
+
+def test_rotary_frequencies():
+    ang = P.rotary_angles(np.array([0, 1, 5]), 8, 10000.0)
+    assert ang.dtype == np.float32 and ang.shape == (3, 4)
+    assert np.all(ang[0] == 0) and ang[1, 0] == 1.0
+    assert np.allclose(ang[1], 10000.0 ** (-np.arange(0, 8, 2) / 8), rtol=1e-6)
+    assert np.allclose(ang[2], 5 * ang[1], rtol=1e-6)
+
+
+def test_rotation_pairs_j_with_j_plus_half_and_turns_counterclockwise():
+    d = 8
+    ang = P.rotary_angles(np.array([3]), d, 100.0)
+    x = np.zeros((1, 1, d))
+    x[0, 0, 1] = 1.0  # the first element of pair (1, 1 + d/2)
+    y = P.apply_rotary(x, ang)[0, 0]
+    a = float(ang[0, 1])
+    want = np.zeros(d)
+    want[1], want[1 + d // 2] = np.cos(a), np.sin(a)
+    assert np.allclose(y, want, atol=1e-12)  # interleaved pairing would put the sine at index 0 or 2
+    x = np.zeros((1, 1, d))
+    x[0, 0, 1 + d // 2] = 1.0
+    y = P.apply_rotary(x, ang)[0, 0]
+    want = np.zeros(d)
+    want[1], want[1 + d // 2] = -np.sin(a), np.cos(a)
+    assert np.allclose(y, want, atol=1e-12)
+
+
+def test_rotation_invariants():
+    d = 16
+    q, k = rng.standard_normal((1, 1, d)), rng.standard_normal((1, 1, d))
+    at = lambda x, p: P.apply_rotary(x, P.rotary_angles(np.array([p]), d, 10000.0))[0, 0]
+    assert np.allclose(at(q, 0), q[0, 0])  # position 0 is the identity
+    r = at(q, 7)
+    assert np.allclose(r[: d // 2] ** 2 + r[d // 2 :] ** 2, q[0, 0, : d // 2] ** 2 + q[0, 0, d // 2 :] ** 2)  # pair norms
+    dots = [at(q, m) @ at(k, n) for m, n in ((5, 2), (13, 10), (103, 100))]
+    assert np.allclose(dots, dots[0], rtol=1e-5)  # only the distance counts
+    assert abs(at(q, 5) @ at(k, 2) - at(q, 2) @ at(k, 5)) > 1e-3  # and its sign
+
+
+# ------------------------------------------------------------------------------------------ attention
+
+
+def sdpa(q, k, v, scale, causal):
+    t = lambda x: torch.from_numpy(x).permute(1, 0, 2)[None]
+    out = F.scaled_dot_product_attention(t(q), t(k), t(v), is_causal=causal, scale=scale, enable_gqa=True)
+    return out[0].permute(1, 0, 2).numpy()
+
+
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (6, 2), (6, 1), (1, 1)])
+def test_attention_reduces_to_the_library_routine(hq, hkv):
+    T, d = 9, 8
+    q, k, v = rng.standard_normal((T, hq, d)), rng.standard_normal((T, hkv, d)), rng.standard_normal((T, hkv, d))
+    assert np.allclose(P.attention(q, k, v, 0.3), sdpa(q, k, v, 0.3, True), atol=1e-12)
+    # the last query sees every key: no mask at all
+    assert np.allclose(P.attention(q, k, v, 0.3)[-1:], sdpa(q[-1:], k, v, 0.3, False), atol=1e-12)
+
+
+def test_attention_special_cases():
+    d = 8
+    q, k, v = rng.standard_normal((1, 2, d)), rng.standard_normal((1, 1, d)), rng.standard_normal((1, 1, d))
+    assert np.allclose(P.attention(q, k, v, 1.0)[0], np.broadcast_to(v[0], (2, d)))  # one token: o = v
+    T = 6
+    q = rng.standard_normal((T, 1, d))
+    k = np.broadcast_to(rng.standard_normal((1, 1, d)), (T, 1, d)).copy()
+    v = rng.standard_normal((T, 1, d))
+    out = P.attention(q, k, v, 0.7)
+    for t in range(T):
+        assert np.allclose(out[t, 0], v[: t + 1, 0].mean(0))  # equal keys: the mean of the values seen
+    # head h reads KV head h // group
+    hq, hkv = 6, 3
+    q = rng.standard_normal((1, hq, d))
+    k = rng.standard_normal((1, hkv, d))
+    v = np.arange(hkv, dtype=float)[None, :, None] * np.ones((1, hkv, d))
+    assert np.allclose(P.attention(q, k, v, 1.0)[0, :, 0], [0, 0, 1, 1, 2, 2])
+
+
+def test_window_meaning():
+    T, d = 12, 8
+    q, k, v = rng.standard_normal((T, 2, d)), rng.standard_normal((T, 1, d)), rng.standard_normal((T, 1, d))
+    assert np.allclose(P.attention(q, k, v, 0.5, window=T), P.attention(q, k, v, 0.5))
+    assert np.allclose(P.attention(q, k, v, 0.5, window=1), np.broadcast_to(v, (T, 2, d)))  # only itself
+    w3 = P.attention(q, k, v, 0.5, window=3)
+    for t in (2, 7, 11):  # the last three keys, as a short sequence of its own
+        lo = max(0, t - 2)
+        assert np.allclose(w3[t], P.attention(q[lo : t + 1], k[lo : t + 1], v[lo : t + 1], 0.5)[-1])
+
+
+def test_swiglu():
+    x = rng.standard_normal((4, 6))
+    wg, wu, wd = rng.standard_normal((10, 6)), rng.standard_normal((10, 6)), rng.standard_normal((6, 10))
+    g = x @ wg.T
+    assert np.allclose(P.swiglu(x, wg, wu, wd), (g / (1 + np.exp(-g)) * (x @ wu.T)) @ wd.T)
+    assert P.silu(np.zeros(3)).tolist() == [0, 0, 0] and np.isclose(P.silu(np.array([20.0]))[0], 20.0)
+    assert not np.allclose(P.swiglu(x, wg, wu, wd), P.swiglu(x, wu, wg, wd))  # gate and up are not interchangeable
+
+
+# ------------------------------------------------------------------------------------------ the whole model
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("plain")
+    return {n: read_model_folder(write_model_folder(root / n, cfg, seed, init)) for n, (cfg, seed, init) in TINY.items()}
+
+
+@pytest.mark.parametrize("name", sorted(TINY))
+def test_only_distances_between_positions_count(name, models):
+    cfg, w = models[name]
+    ids = rng.integers(0, cfg["vocab_size"], 20)
+    base = P.logits(cfg, w, ids)
+    shifted = P.logits(cfg, w, ids, positions=np.arange(20) + 37)
+    assert np.abs(shifted - base).max() < 2e-4 * np.abs(base).max()  # float32 angles: equal up to their rounding
+    later = np.arange(20)
+    later[10:] += 1  # a gap in the middle is not a shift of all positions
+    assert np.abs(P.logits(cfg, w, ids, positions=later)[10:] - base[10:]).max() > 1e-3 * np.abs(base).max()
+
+
+@pytest.mark.parametrize("name", sorted(TINY))
+def test_causality_and_dependence(name, models):
+    cfg, w = models[name]
+    ids = rng.integers(0, cfg["vocab_size"], 40)
+    base = P.logits(cfg, w, ids)
+    other = ids.copy()
+    other[25] = (other[25] + 1) % cfg["vocab_size"]
+    changed = P.logits(cfg, w, other)
+    assert np.array_equal(changed[:25], base[:25])  # a token never changes what came before it
+    assert np.abs(changed[25:] - base[25:]).max() > 1e-6
+    assert np.allclose(P.logits(cfg, w, ids[:17]), base[:17], rtol=0, atol=1e-12)  # a prefix is a prefix
+
+
+def test_window_layers_forget_far_tokens(models):
+    cfg, w = models["tinyC"]  # window 24 in layers 0, 2, 3; layer 1 sees everything
+    ids = rng.integers(0, cfg["vocab_size"], 60)
+    base = P.logits(cfg, w, ids)
+    other = ids.copy()
+    other[3] = (other[3] + 1) % cfg["vocab_size"]
+    assert np.abs(P.logits(cfg, w, other)[-1] - base[-1]).max() > 1e-9  # the full layer still carries it
+    # four windowed layers of window 6 reach back at most 4 * 5 tokens
+    short = dict(cfg, sliding_window=6, layer_types=["sliding_attention"] * 4)
+    a, b = P.logits(short, w, ids), P.logits(short, w, other)
+    assert np.array_equal(a[3 + 4 * 5 + 1 :], b[3 + 4 * 5 + 1 :]) and not np.array_equal(a[3 : 3 + 4 * 5 + 1], b[3 : 3 + 4 * 5 + 1])
+
+
+def test_tied_and_untied_heads(models):
+    cfg_a, w_a = models["tinyA"]
+    assert cfg_a["tie_word_embeddings"] and w_a["lm_head.weight"] is w_a["model.embed_tokens.weight"]
+    cfg_b, w_b = models["tinyB"]
+    assert not cfg_b["tie_word_embeddings"] and not np.array_equal(w_b["lm_head.weight"], w_b["model.embed_tokens.weight"])
+
+
+def test_config_rules():
+    cfg = dict(TINY["tinyA"][0])
+    del cfg["head_dim"]
+    assert P.read_config(cfg)["D"] == 16
+    for key, val in (("rope_scaling", {"factor": 2}), ("hidden_act", "gelu")):
+        with pytest.raises(NotImplementedError):
+            P.read_config(dict(cfg, **{key: val}))
+
+
+# ------------------------------------------------------------------------------------------ sampling
+
+
+def test_greedy_takes_the_first_maximum():
+    row = np.zeros(40)
+    row[[3, 7]] = 5.0
+    assert P.sample(row, 0.0, 1, 1) == 3
+    row[[30, 5]] = 9.0
+    assert P.sample(row, 0.0, 1, 1) == 5
+
+
+def test_noise_is_uniform_keyed_and_pure():
+    u = P.uniform_noise(123, 45, 20000)
+    assert u.min() > 0 and u.max() < 1 and abs(u.mean() - 0.5) < 0.01
+    assert np.array_equal(u, P.uniform_noise(123, 45, 20000))
+    assert not np.array_equal(u, P.uniform_noise(124, 45, 20000)) and not np.array_equal(u, P.uniform_noise(123, 46, 20000))
+    assert np.array_equal(u[:100], P.uniform_noise(123, 45, 100))  # entry v does not depend on the vocabulary size
+    assert P.mix32(0) == 0 and P.mix32(1) == P.mix32(1) and 0 <= P.mix32(0xFFFFFFFF) < 2**32
+
+
+def test_temperature_frequencies_follow_softmax():
+    logits = np.array([2, 1, 0.5, 0, -1, -3, 1.5, 0.2])
+    for temp in (0.5, 2.0):
+        draws = [P.sample(logits, temp, seed, 0) for seed in range(4000)]
+        freq = np.bincount(draws, minlength=8) / 4000
+        p = np.exp(logits / temp)
+        assert np.abs(freq - p / p.sum()).max() < 0.03
+
+
+def test_nucleus_keeps_the_smallest_set_reaching_top_p():
+    logits = np.log(np.array([0.5, 0.3, 0.15, 0.05]))
+    assert {P.sample(logits, 1.0, s, 0, top_p=0.5) for s in range(300)} == {0}  # mass before token 1 is 0.5, not < 0.5
+    assert {P.sample(logits, 1.0, s, 0, top_p=0.6) for s in range(300)} == {0, 1}
+    assert {P.sample(logits, 1.0, s, 0, top_p=0.96) for s in range(600)} == {0, 1, 2, 3}
+    tie = np.log(np.array([0.25, 0.25, 0.25, 0.25]))
+    assert {P.sample(tie, 1.0, s, 0, top_p=0.3) for s in range(300)} == {0, 1}  # ties stay in index order
