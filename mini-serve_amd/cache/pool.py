@@ -1,10 +1,11 @@
 """Device storage of the cache: per group one tensor of pages, per stateful slot one tensor of
 state slots.
 
-Pages of a group: ``[slots_in_group, 2 (K, V), pages + 1, kv_heads, page_size, head_dim]`` in the
-compute dtype, zero-initialised. Within a page the tokens of one KV head are contiguous
-(``page_size * head_dim`` elements), so an attention workgroup that owns one KV head streams whole
-contiguous runs per page. (The reference keeps ``[2, layers, blocks, block_size, kv_heads,
+Pages of a group: ``[slots_in_group, 2 (K, V), pages + 1, kv_heads, page_size * head_dim]`` in the
+compute dtype, zero-initialised. One KV head of one page is a contiguous run, so an attention
+workgroup that owns a KV head streams whole runs. Keys lie ``[page_size, head_dim]`` inside the run;
+values lie transposed, ``[head_dim, page_size]``: the tokens of one head element are contiguous,
+which is the order the matrix cores need them in for the probability-value product. (The reference keeps ``[2, layers, blocks, block_size, kv_heads,
 head_dim]``, miniserve/cache/kv_pool.py:32-44.) The one extra page past the allocator's range is
 the dummy page that padding rows of a captured decode graph write to and read from
 (miniserve/engine/model_runner.py:111-113).
@@ -24,7 +25,7 @@ class LayerCache:
     """What a mixer gets for one run-order entry."""
 
     k: torch.Tensor  # [pages + 1, kv_heads, page_size, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor  # [pages + 1, kv_heads, head_dim, page_size]
     block_table: torch.Tensor  # int32 [rows, width] page ids of this group
     slots: torch.Tensor  # int32 [tokens] page * page_size + offset of each new token
     writes: bool
@@ -68,7 +69,9 @@ class KVPool:
         gi, i = where
         gb = batch.groups[gi]
         buf = self.buffers[gi]
-        return LayerCache(buf[i, 0], buf[i, 1], gb.block_table, gb.slots, writes, self.page_size, self.layout.groups[gi].window)
+        g = self.layout.groups[gi]
+        v = buf[i, 1].view(buf.shape[2], g.num_kv_heads, g.head_dim, self.page_size)
+        return LayerCache(buf[i, 0], v, gb.block_table, gb.slots, writes, self.page_size, g.window)
 
     def state_view(self, slot: int, batch):
         return self.states.get(slot)

@@ -1,12 +1,13 @@
 // Causal grouped-query attention over the paged cache, generic form: any head size that is a
 // multiple of 16 up to 256, any head counts, float32 or bfloat16 storage, float32 arithmetic.
 //
-// One wave per (token, query head). Keys are visited in tiles of 64 aligned to absolute positions
+// One wave per (token, query head); ``token_list`` (optional) names the flat token indices to run. Keys are visited in tiles of 64 aligned to absolute positions
 // (tile boundaries at multiples of 64), so what a query computes depends only on its position, the
 // window and the cache contents: not on how tokens were cut into steps or batched.
 //   scores: lane = key; softmax: running maximum and sum (float32); values: lane = head element.
 //
-// Cache layout [pages, Hkv, page_size, D]; block_table[row, i] = page of the row's tokens
+// Cache layouts: keys [pages, Hkv, page_size, D], values [pages, Hkv, D, page_size] (transposed
+// within the page); block_table[row, i] = page of the row's tokens
 // i * page_size .. ; a query at position p of row b sees keys max(0, p - window + 1) .. p
 // (window == 0: all keys 0 .. p). Query head h reads KV head h / (Hq / Hkv).
 #include "common.h"
@@ -20,13 +21,14 @@ template <> struct Vec16<bf16> { static constexpr int N = 8; };
 template <typename T>
 __global__ __launch_bounds__(WAVE) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kc, const T* __restrict__ vc,
-    const int* __restrict__ block_table, int table_width, const int* __restrict__ token_row,
-    const int* __restrict__ pos, T* __restrict__ out, int Hq, int Hkv, int D, int page_size, float scale, int window) {
+    const int* __restrict__ block_table, int table_width, const int* __restrict__ token_list,
+    const int* __restrict__ token_row, const int* __restrict__ pos, T* __restrict__ out, int Hq, int Hkv, int D,
+    int page_size, float scale, int window) {
   __shared__ __attribute__((aligned(16))) float qs[MAX_HEAD_DIM];
   __shared__ float ps[WAVE];
   constexpr int VN = Vec16<T>::N;
   constexpr int PER = MAX_HEAD_DIM / WAVE;
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int kvh = h / (Hq / Hkv);
   const int p = pos[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
@@ -71,12 +73,12 @@ __global__ __launch_bounds__(WAVE) void paged_attention_generic_kernel(
     const int je = j0 + WAVE - 1 < p ? j0 + WAVE - 1 : p;
     for (int jj = jb; jj <= je; ++jj) {
       const int page = table[jj / page_size];
-      const T* vp = vc + (((size_t)page * Hkv + kvh) * page_size + (jj % page_size)) * D;
+      const T* vp = vc + ((size_t)page * Hkv + kvh) * D * page_size + (jj % page_size);
       const float w = ps[jj - j0];
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int e = lane + i * WAVE;
-        if (e < D) o[i] = fmaf(w, to_f32(vp[e]), o[i]);
+        if (e < D) o[i] = fmaf(w, to_f32(vp[(size_t)e * page_size]), o[i]);
       }
     }
   }
@@ -90,9 +92,9 @@ __global__ __launch_bounds__(WAVE) void paged_attention_generic_kernel(
 }
 
 extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const void* kc, const void* vc, int is_bf16,
-                                          const int* block_table, int table_width, const int* token_row, const int* pos,
-                                          void* out, int tokens, int Hq, int Hkv, int D, int page_size, float scale,
-                                          int window, hipStream_t st) {
+                                          const int* block_table, int table_width, const int* token_list,
+                                          const int* token_row, const int* pos, void* out, int tokens, int Hq, int Hkv,
+                                          int D, int page_size, float scale, int window, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (D <= 0 || D > MAX_HEAD_DIM || D % 16 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 || window < 0 ||
       table_width <= 0 || Hq > 65535 || q_stride < Hq * D)
@@ -100,11 +102,12 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
   dim3 grid(tokens, Hq);
   if (is_bf16)
     paged_attention_generic_kernel<bf16><<<grid, WAVE, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc,
-                                                                block_table, table_width, token_row, pos, (bf16*)out, Hq,
-                                                                Hkv, D, page_size, scale, window);
+                                                                block_table, table_width, token_list, token_row, pos,
+                                                                (bf16*)out, Hq, Hkv, D, page_size, scale, window);
   else
     paged_attention_generic_kernel<float><<<grid, WAVE, 0, st>>>((const float*)q, q_stride, (const float*)kc,
-                                                                 (const float*)vc, block_table, table_width, token_row,
-                                                                 pos, (float*)out, Hq, Hkv, D, page_size, scale, window);
+                                                                 (const float*)vc, block_table, table_width, token_list,
+                                                                 token_row, pos, (float*)out, Hq, Hkv, D, page_size, scale,
+                                                                 window);
   return launch_status();
 }

@@ -1,0 +1,222 @@
+// Decode attention for bfloat16: one query token per sequence over the paged cache, split over the
+// keys so that a small batch still fills the chip, then a fixed-order reduction of the splits.
+//
+// Cache layouts (one KV head of one page is contiguous):
+//   keys   K [pages, Hkv, page_size = 16, D]     a token's head is a row of D
+//   values V [pages, Hkv, D, page_size = 16]     transposed within the page: the 16 tokens of one
+//                                                head element are contiguous
+// Both feed v_mfma_f32_16x16x32_bf16 straight from global memory with one vector load per lane:
+//   scores  S^T[token, query] : A operand = K rows (i = token), B operand = Q (j = query head of the group)
+//   output  O[query, d]       : A operand = P (i = query, k = token), B operand = V^T (j = d, k = token)
+// A lane of the score result holds 4 tokens of one query for each of two pages; the MFMA's k index
+// of the second product is mapped to tokens so that exactly these 8 values are the lane's P operand:
+// probabilities never move between lanes.
+//
+// Grid: (rows * Hkv, splits). A block of 4 waves takes a contiguous range of 32-token chunks; its
+// waves take chunks in turn and are merged in LDS. splits == 1 writes the result directly.
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define PAGE 16
+#define CHUNK 32  // tokens per step of a wave: two pages
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_width, const int* __restrict__ tokens,
+    const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int Hq, int Hkv, float scale, int window) {
+  constexpr int KK = D / 32;  // k-steps of the score product
+  constexpr int DB = D / 16;  // 16-wide blocks of the head
+  const int G = Hq / Hkv;
+  const int b = blockIdx.x / Hkv, kvh = blockIdx.x % Hkv;
+  const int split = blockIdx.y, splits = gridDim.y;
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int tok = tokens ? tokens[b] : b;
+  const int kv_len = pos[tok] + 1;
+  const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
+  const int lo_al = lo & ~(CHUNK - 1);
+  const int n_chunks = (kv_len - lo_al + CHUNK - 1) / CHUNK;
+  const int per = (n_chunks + splits - 1) / splits;
+  const int c_begin = split * per;
+  const int c_end = min(n_chunks, c_begin + per);
+  const int* table = block_table + (size_t)token_row[tok] * table_width;
+
+  // Query operand: column r is query head kvh * G + r of the group (zero beyond the group).
+  bf16x8 qf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    if (r < G) {
+      qf[kk] = *reinterpret_cast<const bf16x8*>(q + (size_t)tok * q_stride + (size_t)(kvh * G + r) * D + kk * 32 + g * 8);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[kk][i] = static_cast<bf16>(0.f);
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;  // of query r (replicated over the four lane groups)
+  floatx4 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int c = c_begin + wave; c < c_end; c += 4) {
+    const int t0 = lo_al + c * CHUNK;
+    int p0 = table[t0 / PAGE];
+    int p1 = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0;
+    p0 = max(p0, 0);  // a page behind the window was given back: its tokens are masked below
+    p1 = max(p1, 0);
+    const bf16* k0 = kc + (((size_t)p0 * Hkv + kvh) * PAGE + r) * D + g * 8;
+    const bf16* k1 = kc + (((size_t)p1 * Hkv + kvh) * PAGE + r) * D + g * 8;
+    bf16x8 ka[KK], kb[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      ka[kk] = *reinterpret_cast<const bf16x8*>(k0 + kk * 32);
+      kb[kk] = *reinterpret_cast<const bf16x8*>(k1 + kk * 32);
+    }
+    // V^T operand: element d = db * 16 + r, tokens 4 g .. 4 g + 3 of each page.
+    const bf16* v0 = vc + (((size_t)p0 * Hkv + kvh) * D + r) * PAGE + g * 4;
+    const bf16* v1 = vc + (((size_t)p1 * Hkv + kvh) * D + r) * PAGE + g * 4;
+    bf16x4 va[DB], vb[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      va[db] = *reinterpret_cast<const bf16x4*>(v0 + (size_t)db * 16 * PAGE);
+      vb[db] = *reinterpret_cast<const bf16x4*>(v1 + (size_t)db * 16 * PAGE);
+    }
+    floatx4 s0 = floatx4{0.f, 0.f, 0.f, 0.f}, s1 = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], qf[kk], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[kk], qf[kk], s1, 0, 0, 0);
+    }
+    // This lane: tokens t0 + 4 g + i (s0) and t0 + 16 + 4 g + i (s1) of query r.
+    float sc[8];
+    float m_new = m_run;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ta = t0 + 4 * g + i, tb = ta + PAGE;
+      sc[i] = (ta >= lo && ta < kv_len) ? s0[i] * scale : -INFINITY;
+      sc[4 + i] = (tb >= lo && tb < kv_len) ? s1[i] * scale : -INFINITY;
+      m_new = fmaxf(m_new, fmaxf(sc[i], sc[4 + i]));
+    }
+    m_new = fmaxf(m_new, __shfl_xor(m_new, 16, WAVE));
+    m_new = fmaxf(m_new, __shfl_xor(m_new, 32, WAVE));
+    // A chunk that holds no visible token at all cannot occur: chunks start at the window's first
+    // token's chunk and end at the last token's.
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = expf(sc[i] - m_new);
+      psum += p;
+      pf[i] = static_cast<bf16>(p);
+    }
+    psum += __shfl_xor(psum, 16, WAVE);
+    psum += __shfl_xor(psum, 32, WAVE);
+    const float corr = expf(m_run - m_new);
+    l_run = l_run * corr + psum;
+    m_run = m_new;
+    // Output rows are queries 4 g + i: fetch their correction from the lanes that own those queries.
+    float cq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) cq[i] = __shfl(corr, 4 * g + i, WAVE);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] *= cq[i];
+      bf16x8 vf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        vf[i] = va[db][i];
+        vf[4 + i] = vb[db][i];
+      }
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+    }
+  }
+
+  // Merge the block's four waves: per query (m, l) and O[query][D].
+  __shared__ float sm[4][16], sl[4][16];
+  __shared__ float so[4][16][D + 1];
+  if (g == 0) {
+    sm[wave][r] = m_run;
+    sl[wave][r] = l_run;
+  }
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) so[wave][4 * g + i][db * 16 + r] = o[db][i];
+  __syncthreads();
+  for (int e = tid; e < G * D; e += 256) {
+    const int qh = e / D, d = e % D;
+    float M = fmaxf(fmaxf(sm[0][qh], sm[1][qh]), fmaxf(sm[2][qh], sm[3][qh]));
+    float L = 0.f, O = 0.f;
+    if (M > -INFINITY) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float f = expf(sm[w][qh] - M);  // 0 for a wave that saw nothing
+        L += sl[w][qh] * f;
+        O += so[w][qh][d] * f;
+      }
+    }
+    const int head = kvh * G + qh;
+    if (splits == 1) {
+      out[((size_t)tok * Hq + head) * D + d] = static_cast<bf16>(O / L);
+    } else {
+      const size_t at = ((size_t)b * Hq + head) * splits + split;
+      part_o[at * D + d] = O;
+      if (d == 0) {
+        part_ml[at * 2] = M;
+        part_ml[at * 2 + 1] = L;
+      }
+    }
+  }
+}
+
+// Reduction of the splits in ascending order: grid (rows, Hq), D threads.
+template <int D>
+__global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                const int* __restrict__ tokens, bf16* __restrict__ out,
+                                                                int Hq, int splits) {
+  const int b = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  const size_t base = ((size_t)b * Hq + head) * splits;
+  float M = -INFINITY;
+  for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  float L = 0.f, O = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float m = part_ml[(base + s) * 2];
+    if (m == -INFINITY) continue;  // an empty split
+    const float f = expf(m - M);
+    L += part_ml[(base + s) * 2 + 1] * f;
+    O += part_o[(base + s) * D + d] * f;
+  }
+  const int tok = tokens ? tokens[b] : b;
+  out[((size_t)tok * Hq + head) * D + d] = static_cast<bf16>(O / L);
+}
+
+// rows decode tokens (tokens[i] = flat token index, or nullptr for the identity). part_o holds
+// rows * Hq * splits * D floats, part_ml rows * Hq * splits * 2 (unused when splits == 1).
+extern "C" int ms_attention_decode_bf16(const void* q, int q_stride, const void* kc, const void* vc,
+                                        const int* block_table, int table_width, const int* tokens,
+                                        const int* token_row, const int* pos, void* out, float* part_o, float* part_ml,
+                                        int rows, int splits, int Hq, int Hkv, int D, int page_size, float scale,
+                                        int window, hipStream_t st) {
+  if (rows <= 0) return MS_OK;
+  if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || splits < 1 || splits > 65535 || window < 0 || table_width <= 0 ||
+      q_stride < Hq * D || q_stride % 8 || (splits > 1 && (!part_o || !part_ml)))
+    return MS_BAD_ARG;
+  dim3 grid(rows * Hkv, splits);
+#define LAUNCH(DD)                                                                                                     \
+  attn_decode_split_kernel<DD><<<grid, 256, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc,       \
+                                                     block_table, table_width, tokens, token_row, pos, (bf16*)out,    \
+                                                     part_o, part_ml, Hq, Hkv, scale, window);                         \
+  if (splits > 1)                                                                                                      \
+    attn_decode_reduce_kernel<DD><<<dim3(rows, Hq), DD, 0, st>>>(part_o, part_ml, tokens, (bf16*)out, Hq, splits)
+  if (D == 128) { LAUNCH(128); } else { LAUNCH(64); }
+#undef LAUNCH
+  return launch_status();
+}

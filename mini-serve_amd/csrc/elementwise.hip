@@ -98,7 +98,8 @@ extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf1
 //   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
 //         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j];
 //   q is written back in place; k and v go to the cache page of the token's slot
-//   (cache layout [pages, Hkv, page_size, D]; slot = page * page_size + offset).
+//   (slot = page * page_size + offset; keys [pages, Hkv, page_size, D], values transposed within
+//   the page, [pages, Hkv, D, page_size]).
 // With slots == nullptr only the query heads are processed (the entry reads another entry's cache).
 #define MAX_HEAD_DIM 256
 template <typename T, typename TW>
@@ -120,11 +121,14 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const int* __rest
     ss += x[i] * x[i];
   }
   T* dst = src;
-  if (kind != 0) {
+  size_t dst_step = 1;  // distance between consecutive head elements at the destination
+  if (kind == 1) {
     const int s = slots[t];
-    const int kvh = kind == 1 ? hs - Hq : hs - Hq - Hkv;
-    T* base = kind == 1 ? kc : vc;
-    dst = base + (((size_t)(s / page_size) * Hkv + kvh) * page_size + (s % page_size)) * D;
+    dst = kc + (((size_t)(s / page_size) * Hkv + (hs - Hq)) * page_size + (s % page_size)) * D;
+  } else if (kind == 2) {
+    const int s = slots[t];
+    dst = vc + ((size_t)(s / page_size) * Hkv + (hs - Hq - Hkv)) * D * page_size + (s % page_size);
+    dst_step = page_size;
   }
   if (kind != 2) {
     const TW* w = kind == 0 ? qw : kw;
@@ -161,7 +165,7 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const int* __rest
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + i * WAVE;
-    if (e < D) dst[e] = from_f32<T>(x[i]);
+    if (e < D) dst[(size_t)e * dst_step] = from_f32<T>(x[i]);
   }
 }
 

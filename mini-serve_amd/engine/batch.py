@@ -32,11 +32,14 @@ class GroupBatch:
 
 
 class StepBatch:
-    """Device-side description of a step. Built by ``BatchBuilder.build``."""
+    """Device-side description of a step. Built by ``BatchBuilder.build``. ``decode_tokens`` /
+    ``prefill_tokens``: flat indices of the tokens of rows that bring one token / several tokens
+    (None when all tokens are of one kind: the list is then the identity)."""
 
     __slots__ = (
         "num_rows", "num_tokens", "num_wanted", "token_ids", "positions", "token_row", "row_start", "starts",
         "kv_lens", "state_slots", "want_rows", "groups", "row_lens", "row_starts_host", "max_kv_len", "is_decode",
+        "num_decode_tokens", "decode_tokens", "prefill_tokens",
     )
 
 
@@ -80,6 +83,10 @@ class BatchBuilder:
         take("ids", T); take("pos", T); take("row", T)
         take("row_start", B + 1); take("starts", B); take("kv_lens", B); take("state", B)
         take("want", n_want)
+        n_dec = sum(1 for n in lens if n == 1)
+        mixed = 0 < n_dec < B
+        if mixed:
+            take("dec_tok", n_dec); take("pre_tok", T - n_dec)
         for g in range(self.num_groups):
             take(f"slots{g}", T)
             take(f"table{g}", B * widths[g])
@@ -106,6 +113,17 @@ class BatchBuilder:
                 w += 1
             t += n
         row_start[B] = T
+        if mixed:
+            dec, pre = view("dec_tok"), view("pre_tok")
+            t = d = q = 0
+            for n in lens:
+                if n == 1:
+                    dec[d] = t
+                    d += 1
+                else:
+                    pre[q : q + n] = np.arange(t, t + n, dtype=np.int32)
+                    q += n
+                t += n
         view("starts")[:] = starts
         view("kv_lens")[:] = [s + n for s, n in zip(starts, lens)]
         view("state")[:] = [r.cache.state_slot if r.cache.state_slot is not None else 0 for r in rows]
@@ -135,5 +153,9 @@ class BatchBuilder:
         b.row_lens = lens
         b.row_starts_host = list(starts)
         b.max_kv_len = max(s + n for s, n in zip(starts, lens))
-        b.is_decode = all(n == 1 for n in lens)
+        b.is_decode = n_dec == B
+        b.num_decode_tokens = n_dec
+        # None stands for the identity list (every token is one)
+        b.decode_tokens = dview("dec_tok") if mixed else None
+        b.prefill_tokens = dview("pre_tok") if mixed else None
         return b

@@ -63,7 +63,13 @@ class ModelRunner:
         self.cache = CacheManager(self.layout, page_size, per_group, max_running, max_step_tokens, **kw)
         self.pool = KVPool(self.layout, page_size, per_group, max_running, model.dtype, self.device)
         self.builder = BatchBuilder(self.device, len(self.layout.groups))
+        self.graphs = None
+        if decode_graph and self.device.type == "cuda":
+            from .graphs import DecodeGraphs
+
+            self.graphs = DecodeGraphs(self, decode_graph_max_bs or max_running)
         self.steps = 0
+        self.graph_steps = 0
 
     def _pages_that_fit(self, per_page: int, fraction: float, step_tokens: int) -> int | None:
         if self.device.type != "cuda" or per_page == 0:
@@ -112,8 +118,12 @@ class ModelRunner:
         starts = [r.cache.num_tokens for r in rows]
         for r in rows:
             self.cache.extend(r.cache, len(r.tokens))
-        batch = self.builder.build(rows, starts)
-        logits = self.model.forward(batch, self.pool)
+        if self.graphs is not None and self.graphs.usable(rows):
+            logits = self.graphs.run(rows, starts)
+            self.graph_steps += 1
+        else:
+            batch = self.builder.build(rows, starts)
+            logits = self.model.forward(batch, self.pool)
         for r in rows:
             self.cache.advance(r.cache)
         self.steps += 1

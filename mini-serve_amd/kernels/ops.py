@@ -30,7 +30,9 @@ _SIGNATURES = {
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
-                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
+                                 _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
 }
 
@@ -213,11 +215,7 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
         _dev(slots, "slots", I32, 1)
         if slots.shape[0] != t:
             raise ValueError("one slot per token is needed")
-        for c, nm in ((k_cache, "k_cache"), (v_cache, "v_cache")):
-            _dev(c, nm, qkv.dtype, 4)
-            if c.shape[1] != num_kv_heads or c.shape[3] != head_dim:
-                raise ValueError(f"{nm} is {tuple(c.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
-        page_size = k_cache.shape[2]
+        page_size = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
     if inv_freq is not None:
         _dev(inv_freq, "inv_freq", F32, 1)
         if rot_dim % 2 or rot_dim > head_dim or inv_freq.shape[0] != rot_dim // 2:
@@ -231,15 +229,39 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
         "qk_norm_rope_store")
 
 
+def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
+    """Keys ``[pages, Hkv, page, D]``, values ``[pages, Hkv, D, page]``; returns the page size."""
+    _dev(k_cache, "k_cache", dtype, 4)
+    _dev(v_cache, "v_cache", dtype, 4)
+    page = k_cache.shape[2]
+    if tuple(k_cache.shape[1:]) != (num_kv_heads, page, head_dim):
+        raise ValueError(f"k_cache is {tuple(k_cache.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
+    if tuple(v_cache.shape) != (k_cache.shape[0], num_kv_heads, head_dim, page):
+        raise ValueError(f"v_cache is {tuple(v_cache.shape)}, expected [{k_cache.shape[0]}, {num_kv_heads}, {head_dim}, {page}]")
+    return page
+
+
+DECODE_TARGET_BLOCKS = 512  # workgroups the split decode kernel aims for
+DECODE_MIN_CHUNKS = 4  # 32-token chunks a split should at least hold
+
+
+def decode_splits(rows: int, num_kv_heads: int, max_kv_len: int) -> int:
+    """How many ways the keys of each sequence are split in the decode kernel: enough workgroups to
+    fill the chip, but no split shorter than a few chunks."""
+    by_fill = -(-DECODE_TARGET_BLOCKS // max(1, rows * num_kv_heads))
+    by_len = max(1, -(-max_kv_len // 32) // DECODE_MIN_CHUNKS)
+    return max(1, min(by_fill, by_len))
+
+
 def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window):
     """Attention of the batch's new tokens over the cache. ``qkv [T, >= Hq D]`` holds the queries
-    in its first ``Hq * D`` columns. Returns ``[T, Hq * D]``."""
+    in its first ``Hq * D`` columns. Returns ``[T, Hq * D]``.
+
+    bfloat16 with 16-token pages and a head size of 64 or 128: rows that bring one token run the
+    split decode kernel. Everything else runs the generic kernel."""
     _dev(qkv, "qkv", (F32, BF16), 2)
     t = qkv.shape[0]
-    for c, nm in ((k_cache, "k_cache"), (v_cache, "v_cache")):
-        _dev(c, nm, qkv.dtype, 4)
-        if c.shape[1] != num_kv_heads or c.shape[3] != head_dim:
-            raise ValueError(f"{nm} is {tuple(c.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
+    page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
     if head_dim % 16 or not 16 <= head_dim <= 256:
         raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 up to 256")
     if num_heads % num_kv_heads:
@@ -252,11 +274,29 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
         raise ValueError("batch metadata does not match the number of tokens or rows")
     out = torch.empty((t, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    _check(library().ms_paged_attention_generic(
-        qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16),
-        block_table.data_ptr(), block_table.shape[1], batch.token_row.data_ptr(), batch.positions.data_ptr(),
-        out.data_ptr(), t, num_heads, num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), _stream()),
-        "paged_attention")
+    lib = library()
+    common = (block_table.data_ptr(), block_table.shape[1])
+    n_dec = batch.num_decode_tokens
+    fast = (qkv.dtype == BF16 and page == 16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 16
+            and qkv.shape[1] % 8 == 0)
+    if fast and n_dec:
+        splits = decode_splits(n_dec, num_kv_heads, batch.max_kv_len)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty((n_dec * num_heads * splits * head_dim,), dtype=F32, device=qkv.device)
+            part_ml = torch.empty((n_dec * num_heads * splits * 2,), dtype=F32, device=qkv.device)
+        _check(lib.ms_attention_decode_bf16(
+            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, _ptr(batch.decode_tokens),
+            batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml), n_dec,
+            splits, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_decode")
+        rest, n_rest = batch.prefill_tokens, t - n_dec
+    else:
+        rest, n_rest = None, t
+    if n_rest:
+        _check(lib.ms_paged_attention_generic(
+            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common,
+            _ptr(rest), batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), n_rest, num_heads,
+            num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "paged_attention")
     return out
 
 

@@ -147,7 +147,7 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
     slots = perm.to(torch.int32).to(DEV)
     inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
     kc = torch.full((pages, hkv, page, d), 7.0, dtype=dtype, device=DEV)
-    vc = torch.full((pages, hkv, page, d), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, hkv, d, page), 7.0, dtype=dtype, device=DEV)  # values lie transposed within the page
     ref = qkv.double().view(t, hq + 2 * hkv, d)
     q, k, v = ref[:, :hq], ref[:, hq : hq + hkv], ref[:, hq + hkv :]
 
@@ -162,7 +162,7 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
     close(work.view(t, hq + 2 * hkv, d)[:, :hq], qn, tol, "q")
     sl = slots.long()
     got_k = kc.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)
-    got_v = vc.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)
+    got_v = vc.permute(0, 3, 1, 2).reshape(pages * page, hkv, d)
     close(got_k[sl], kn, tol, "k in cache")
     assert torch.equal(got_v[sl].double(), v), "v is stored as it is"
     untouched = torch.ones(pages * page, dtype=torch.bool)
@@ -176,8 +176,29 @@ class _Batch:
     pass
 
 
-def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=0):
-    """Rows with ``starts[i]`` cached tokens and ``lens_new[i]`` new ones; scattered pages."""
+def make_batch(lens_new, starts):
+    batch = _Batch()
+    batch.num_rows = len(lens_new)
+    batch.token_row = torch.tensor([i for i, n in enumerate(lens_new) for _ in range(n)], dtype=torch.int32, device=DEV)
+    batch.positions = torch.tensor([s + j for s, n in zip(starts, lens_new) for j in range(n)], dtype=torch.int32, device=DEV)
+    batch.max_kv_len = max(s + n for s, n in zip(starts, lens_new))
+    n_dec = sum(1 for n in lens_new if n == 1)
+    batch.num_decode_tokens = n_dec
+    batch.decode_tokens = batch.prefill_tokens = None
+    if 0 < n_dec < len(lens_new):
+        dec, pre, t = [], [], 0
+        for n in lens_new:
+            (dec if n == 1 else pre).extend(range(t, t + n))
+            t += n
+        batch.decode_tokens = torch.tensor(dec, dtype=torch.int32, device=DEV)
+        batch.prefill_tokens = torch.tensor(pre, dtype=torch.int32, device=DEV)
+    return batch
+
+
+def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=0, boost=None):
+    """Rows with ``starts[i]`` cached tokens and ``lens_new[i]`` new ones; scattered pages.
+    ``boost = (row, position)``: the key there and the row's last query are scaled so that this
+    one score stands out among all others (a far key that is skipped or misplaced then shows)."""
     g = torch.Generator().manual_seed(seed)
     b = len(lens_new)
     totals = [s + n for s, n in zip(starts, lens_new)]
@@ -187,17 +208,21 @@ def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=
     width = max(blocks)
     table = torch.full((b, width), -1, dtype=torch.int32)
     kc = rand((pages, hkv, page, d), dtype, seed + 1)
-    vc = rand((pages, hkv, page, d), dtype, seed + 2)
+    vc = rand((pages, hkv, d, page), dtype, seed + 2)
     at = 0
     for i, nb in enumerate(blocks):
         table[i, :nb] = torch.tensor(order[at : at + nb], dtype=torch.int32)
         at += nb
     t = sum(lens_new)
     q = rand((t, (hq + 2 * hkv) * d), dtype, seed + 3)
-    batch = _Batch()
-    batch.num_rows = b
-    batch.token_row = torch.tensor([i for i, n in enumerate(lens_new) for _ in range(n)], dtype=torch.int32, device=DEV)
-    batch.positions = torch.tensor([s + j for s, n in zip(starts, lens_new) for j in range(n)], dtype=torch.int32, device=DEV)
+    if boost is not None:
+        row, where = boost
+        last = sum(lens_new[: row + 1]) - 1
+        key = kc[table[row, where // page], :, where % page]  # [hkv, d]
+        qv = q[last].view(hq + 2 * hkv, d)
+        for h in range(hq):
+            qv[h] = (key[h // (hq // hkv)].float() * 3.0).to(dtype)
+    batch = make_batch(lens_new, starts)
     scale = d**-0.5
     got = ops.paged_attention(q, kc, vc, table.to(DEV), batch, hq, hkv, d, scale, window)
     want = torch.empty((t, hq, d), dtype=torch.float64)
@@ -206,7 +231,7 @@ def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=
     tok = 0
     for i in range(b):
         keys = torch.stack([kcd[table[i, p // page], :, p % page] for p in range(totals[i])])  # [len, hkv, d]
-        vals = torch.stack([vcd[table[i, p // page], :, p % page] for p in range(totals[i])])
+        vals = torch.stack([vcd[table[i, p // page], :, :, p % page] for p in range(totals[i])])
         for j in range(lens_new[i]):
             p = starts[i] + j
             lo = max(0, p - window + 1) if window else 0
@@ -214,6 +239,8 @@ def attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window, seed=
                 kh = h // (hq // hkv)
                 s = (keys[lo : p + 1, kh] @ qd[tok, h]) * scale
                 w = torch.softmax(s, 0)
+                if boost is not None and boost[0] == i and j == lens_new[i] - 1 and lo <= boost[1] <= p:
+                    assert float(w[boost[1] - lo]) > 0.9, "the boosted key was meant to dominate"
                 want[tok, h] = w @ vals[lo : p + 1, kh]
             tok += 1
     close(got.view(t, hq, d), want, 2e-6 if dtype == F32 else 8e-3, f"attention {hq}/{hkv}/{d} window {window}")
@@ -235,30 +262,46 @@ def test_paged_attention(ops, dtype, hq, hkv, d, page, lens_new, starts, window)
     attention_case(ops, dtype, hq, hkv, d, page, lens_new, starts, window)
 
 
+@pytest.mark.parametrize(
+    "hq,hkv,d,lens_new,starts,window,boost",
+    [
+        (16, 8, 128, [1] * 7, [0, 15, 16, 31, 32, 1000, 4095], 0, None),   # page and chunk edges, many splits
+        (16, 8, 128, [1, 1], [700, 3000], 0, (1, 37)),                     # a far key among thousands
+        (16, 8, 128, [1, 1], [700, 3000], 0, (0, 699)),                    # the newest cached key
+        (32, 8, 128, [1] * 3, [5, 260, 90], 0, (1, 255)),
+        (64, 8, 128, [1] * 2, [513, 77], 0, None),
+        (14, 2, 64, [1] * 5, [63, 64, 65, 2000, 1], 0, (3, 1024)),
+        (6, 6, 64, [1] * 4, [300, 40, 41, 1200], 100, (0, 201)),           # the window's first key
+        (16, 8, 128, [1] * 3, [500, 31, 2047], 33, (2, 2047 - 33 + 1)),
+        (16, 8, 128, [1, 20, 1, 5, 1], [100, 0, 1999, 30, 0], 0, (2, 3)),  # decode rows beside portions
+        (4, 2, 128, [1] * 64, list(range(0, 6400, 100)), 0, None),         # a full batch: one split
+    ],
+)
+def test_decode_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost):
+    attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=30, boost=boost)
+
+
+def test_decode_splits_rule(ops):
+    assert ops.decode_splits(1, 8, 4096) == 32 and ops.decode_splits(8, 8, 4096) == 8 and ops.decode_splits(64, 8, 4096) == 1
+    assert ops.decode_splits(1, 8, 100) == 1 and ops.decode_splits(1, 1, 40000) == 312 and ops.decode_splits(1, 8, 1) == 1
+
+
 def test_attention_one_token_returns_its_value(ops):
     """A sequence of one token: softmax over one key is 1, so the output is v."""
     hq, hkv, d, page = 4, 2, 32, 16
     q = rand((1, (hq + 2 * hkv) * d), F32, 20)
-    kc, vc = rand((2, hkv, page, d), F32, 21), rand((2, hkv, page, d), F32, 22)
-    batch = _Batch()
-    batch.num_rows = 1
-    batch.token_row = torch.zeros(1, dtype=torch.int32, device=DEV)
-    batch.positions = torch.zeros(1, dtype=torch.int32, device=DEV)
+    kc, vc = rand((2, hkv, page, d), F32, 21), rand((2, hkv, d, page), F32, 22)
     table = torch.tensor([[1]], dtype=torch.int32, device=DEV)
-    out = ops.paged_attention(q, kc, vc, table, batch, hq, hkv, d, d**-0.5, 0).view(hq, d)
+    out = ops.paged_attention(q, kc, vc, table, make_batch([1], [0]), hq, hkv, d, d**-0.5, 0).view(hq, d)
     for h in range(hq):
-        assert torch.equal(out[h], vc[1, h // 2, 0])
+        assert torch.equal(out[h], vc[1, h // 2, :, 0])
 
 
 def test_attention_refuses_unsupported_head_size(ops):
     q = rand((1, 3 * 24), F32, 23)
-    kc = rand((1, 1, 16, 24), F32, 24)
-    batch = _Batch()
-    batch.num_rows = 1
-    batch.token_row = torch.zeros(1, dtype=torch.int32, device=DEV)
-    batch.positions = torch.zeros(1, dtype=torch.int32, device=DEV)
+    kc, vc = rand((1, 1, 16, 24), F32, 24), rand((1, 1, 24, 16), F32, 24)
     with pytest.raises(ValueError, match="head_dim 24"):
-        ops.paged_attention(q, kc, kc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), batch, 1, 1, 24, 1.0, 0)
+        ops.paged_attention(q, kc, vc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), make_batch([1], [0]), 1, 1, 24, 1.0, 0)
 
 
 # ------------------------------------------------------------------------------------------ sampling
