@@ -71,10 +71,14 @@ def main() -> int:
         """Decode ``warmup + steps`` tokens for ``batch`` requests ending at the context length;
         returns (seconds for the timed steps, mean context over them, engine)."""
         total = warmup + steps
-        plen = args.context - total
-        eng = Engine(model, max_running=batch, kv_pool_tokens=batch * (args.context + 16), chunked_prefill_size=2048,
+        # Decoding requests keep decoding while later ones are still prefilled (about two steps per
+        # request at a step budget of 2,048 tokens): prompts are shortened by that much, so that the
+        # longest sequence ends at the context length.
+        lead = 2 * batch
+        plen = args.context - total - lead
+        eng = Engine(model, max_running=batch, kv_pool_tokens=batch * (args.context + 32), chunked_prefill_size=2048,
                      decode_graph=not args.no_graph)
-        reqs = [eng.add_request(p, SamplingParams(max_new_tokens=total + 1)) for p in prompts(batch, plen)]
+        reqs = [eng.add_request(p, SamplingParams(max_new_tokens=total + lead + 8)) for p in prompts(batch, plen)]
         say(f"batch {batch}: prefilling {batch} x {plen} tokens")
         last = time.time()
         while not all(r.state is RequestState.DECODE for r in reqs):
@@ -82,17 +86,18 @@ def main() -> int:
             if time.time() - last > 20:
                 last = time.time()
                 say(f"  prefill: {sum(r.cache.num_tokens for r in reqs if r.cache)} tokens in the cache")
-        say(f"batch {batch}: decoding {warmup} + {steps} steps")
-        for _ in range(warmup - 1):  # the step that finished the last prefill produced the first token
+        say(f"batch {batch}: decoding {warmup} + {steps} steps at contexts {min(r.seq_len for r in reqs)}..{max(r.seq_len for r in reqs)}")
+        for _ in range(warmup):
             eng.step()
         torch.cuda.synchronize()
+        ctx0 = sum(r.seq_len for r in reqs) / batch
         t0 = time.perf_counter()
         for _ in range(steps):
             eng.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        first_ctx = reqs[0].seq_len - steps
-        mean_ctx = first_ctx + (steps - 1) / 2
+        assert all(r.state is RequestState.DECODE for r in reqs), "a request ended inside the timed steps"
+        mean_ctx = ctx0 + (steps - 1) / 2
         for r in reqs:
             eng.abort(r.rid)
         return dt, mean_ctx, eng

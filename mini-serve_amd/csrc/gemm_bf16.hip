@@ -210,6 +210,95 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16* __res
   for (int i = 0; i < MB; ++i) store4(C, mode, i * 16 + r, nb + g * 4, M, N, ldc, acc[i], vec_store);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Small-M kernel: M <= 16 rows of X (a decode step of a small batch). No LDS, no barriers: a wave owns
+// 16 weight rows and a slice of K; per step of 64 k each lane loads 32 bytes of its weight row and
+// the matching 32 bytes of an X row (X is a few KB and stays in the vector cache), and issues two
+// MFMAs. K is split over blockIdx.y so that even a 1024-row matrix gives every CU several waves;
+// each split writes float partial sums P[split, M, N], summed afterwards in ascending split order.
+// The number of splits depends on N and K alone, never on M: a row's result does not depend on
+// the batch it is in.
+#define SMALL_UNROLL 4
+
+__global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                              float* __restrict__ P, int M, int N, int K, int ldx,
+                                                              int steps_per_split) {
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int nb = (blockIdx.x * 4 + wave) * 16;
+  if (nb >= N) return;
+  const int n = nb + r;
+  const int k_begin = blockIdx.y * steps_per_split * 64;
+  const int k_end = min(K, k_begin + steps_per_split * 64);
+  const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
+
+  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_begin; k0 < k_end; k0 += 64 * SMALL_UNROLL) {
+    Chunk w[SMALL_UNROLL][2], x[SMALL_UNROLL][2];
+#pragma unroll
+    for (int u = 0; u < SMALL_UNROLL; ++u) {
+      const int k = k0 + u * 64 + g * 16;  // beyond k_end only where k_end == K: load_chunk zero-fills
+      const int kw = k < k_end ? k : K;
+      w[u][0] = load_chunk(W, n, N, kw, K, K, vecw);
+      w[u][1] = load_chunk(W, n, N, kw + 8, K, K, vecw);
+      x[u][0] = load_chunk(X, r, M, kw, K, ldx, vecx);
+      x[u][1] = load_chunk(X, r, M, kw + 8, K, ldx, vecx);
+    }
+#pragma unroll
+    for (int u = 0; u < SMALL_UNROLL; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, x[u][0].v, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, x[u][1].v, acc, 0, 0, 0);
+    }
+  }
+  // acc[i] = C[m = r][n = nb + 4 g + i]
+  float* dst = P + (size_t)blockIdx.y * M * N;
+  store4(dst, 1, r, nb + g * 4, M, N, N, acc, N % 4 == 0);
+}
+
+// C (mode 0 bf16 / 1 float / 2 float +=) from the partial sums, in ascending split order.
+__global__ void splitk_reduce_kernel(const float* __restrict__ P, void* __restrict__ C, int mode, int splits, int M,
+                                     int N, int ldc) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x, m = blockIdx.y;
+  if (n >= N) return;
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += P[((size_t)s * M + m) * N + n];
+  const size_t at = (size_t)m * ldc + n;
+  if (mode == 0) ((bf16*)C)[at] = static_cast<bf16>(v);
+  else if (mode == 1) ((float*)C)[at] = v;
+  else ((float*)C)[at] += v;
+}
+
+// Splits of K for the small-M kernel: enough waves to fill the chip, at least two 64-k steps each.
+extern "C" int ms_gemm_bf16_small_splits(int N, int K) {
+  const int steps = (K + 63) / 64;
+  const int row_blocks = (N + 15) / 16;
+  int want = (1024 + row_blocks - 1) / row_blocks;
+  int most = steps / 2 > 0 ? steps / 2 : 1;
+  int s = want < most ? want : most;
+  if (s < 1) s = 1;
+  const int per = (steps + s - 1) / s;
+  return (steps + per - 1) / per;  // no empty split
+}
+
+// X [M <= 16, K] * W [N, K]^T. `partials` holds splits * M * N floats (splits from
+// ms_gemm_bf16_small_splits). With reduce != 0 the partial sums are folded into C here; otherwise the
+// caller's next kernel sums them.
+extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials, void* C, int mode, int reduce, int M,
+                                  int N, int K, int ldx, int ldc, hipStream_t st) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (M > 16 || K <= 0 || ldx < K || partials == nullptr) return MS_BAD_ARG;
+  const int splits = ms_gemm_bf16_small_splits(N, K);
+  const int steps = (K + 63) / 64;
+  const int per = (steps + splits - 1) / splits;
+  dim3 grid((N + 63) / 64, splits);
+  gemm_bf16_small_kernel<<<grid, 256, 0, st>>>((const bf16*)X, (const bf16*)W, partials, M, N, K, ldx, per);
+  if (reduce) {
+    if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
+    splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);
+  }
+  return launch_status();
+}
+
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
 extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,
                             hipStream_t st) {

@@ -39,8 +39,21 @@ class StepBatch:
     __slots__ = (
         "num_rows", "num_tokens", "num_wanted", "token_ids", "positions", "token_row", "row_start", "starts",
         "kv_lens", "state_slots", "want_rows", "groups", "row_lens", "row_starts_host", "max_kv_len", "is_decode",
-        "num_decode_tokens", "decode_tokens", "prefill_tokens",
+        "num_decode_tokens", "decode_tokens", "prefill_tokens", "_tiles",
     )
+
+    def prefill_tiles(self, tile_tokens: int):
+        """Tiles of at most ``tile_tokens`` consecutive new tokens of the rows that bring several
+        tokens: ``(first flat token index [n], token count [n], n)`` on the device, heaviest
+        (deepest into its sequence) first. Built once per tile size and step."""
+        cache = getattr(self, "_tiles", None)
+        if cache is None:
+            cache = self._tiles = {}
+        if tile_tokens not in cache:
+            from ..kernels.ops import build_prefill_tiles
+
+            cache[tile_tokens] = build_prefill_tiles(self.row_lens, self.row_starts_host, tile_tokens, self.token_ids.device)
+        return cache[tile_tokens]
 
 
 def _align(n: int, to: int = 4) -> int:

@@ -29,10 +29,15 @@ _SIGNATURES = {
                               _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16_small_splits": [_c_int, _c_int],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void,
+                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_prefill_tile_tokens": [_c_int],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
 }
 
@@ -150,6 +155,8 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------------- matrix products
 
+SMALL_M = 16  # rows up to which the split-K weight-streaming kernel runs
+
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None) -> torch.Tensor:
     """``x [M, K] @ weight [N, K]^T``. Either returns a new ``[M, N]`` tensor of ``out_dtype``, or adds
@@ -179,8 +186,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
     else:
         xa = cast(x, BF16)
         mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
-        _check(library().ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
-               "gemm_bf16")
+        lib = library()
+        if m <= SMALL_M:
+            splits = lib.ms_gemm_bf16_small_splits(n, k)
+            if splits == 1 and mode == 1:
+                parts, reduce = out, 0  # the single partial sum is the result
+            else:
+                parts, reduce = torch.empty((splits, m, n), dtype=F32, device=x.device), 1
+            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), out.data_ptr(), mode, reduce,
+                                          m, n, k, k, n, _stream()), "gemm_bf16_small")
+        else:
+            _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
+                   "gemm_bf16")
     return out
 
 
@@ -258,7 +275,8 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     in its first ``Hq * D`` columns. Returns ``[T, Hq * D]``.
 
     bfloat16 with 16-token pages and a head size of 64 or 128: rows that bring one token run the
-    split decode kernel. Everything else runs the generic kernel."""
+    split decode kernel, rows that bring several the tiled prefill kernel. Everything else (float32,
+    other head sizes or page sizes) runs the generic kernel."""
     _dev(qkv, "qkv", (F32, BF16), 2)
     t = qkv.shape[0]
     page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
@@ -276,28 +294,48 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     out = torch.empty((t, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     lib = library()
     common = (block_table.data_ptr(), block_table.shape[1])
+    meta = (batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr())
     n_dec = batch.num_decode_tokens
     fast = (qkv.dtype == BF16 and page == 16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 16
             and qkv.shape[1] % 8 == 0)
-    if fast and n_dec:
+    if not fast:
+        _check(lib.ms_paged_attention_generic(
+            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common, None,
+            *meta, t, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "paged_attention")
+        return out
+    if n_dec:
         splits = decode_splits(n_dec, num_kv_heads, batch.max_kv_len)
         part_o = part_ml = None
         if splits > 1:
             part_o = torch.empty((n_dec * num_heads * splits * head_dim,), dtype=F32, device=qkv.device)
             part_ml = torch.empty((n_dec * num_heads * splits * 2,), dtype=F32, device=qkv.device)
         _check(lib.ms_attention_decode_bf16(
-            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, _ptr(batch.decode_tokens),
-            batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml), n_dec,
-            splits, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_decode")
-        rest, n_rest = batch.prefill_tokens, t - n_dec
-    else:
-        rest, n_rest = None, t
-    if n_rest:
-        _check(lib.ms_paged_attention_generic(
-            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common,
-            _ptr(rest), batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), n_rest, num_heads,
-            num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "paged_attention")
+            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, _ptr(batch.decode_tokens), *meta,
+            _ptr(part_o), _ptr(part_ml), n_dec, splits, num_heads, num_kv_heads, head_dim, page, float(scale), int(window),
+            _stream()), "attention_decode")
+    if n_dec < t:
+        first, count, tiles = batch.prefill_tiles(lib.ms_attention_prefill_tile_tokens(num_heads // num_kv_heads))
+        _check(lib.ms_attention_prefill_bf16(
+            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(),
+            tiles, *meta, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_prefill")
     return out
+
+
+def build_prefill_tiles(row_lens, row_starts, tile_tokens: int, device):
+    """Tiles of at most ``tile_tokens`` consecutive new tokens of the rows that bring several tokens:
+    ``(first flat token index [n], token count [n], n)`` on the device, the tile deepest into its
+    sequence (the most keys to visit) first."""
+    tiles = []
+    t = 0
+    for n, s in zip(row_lens, row_starts):
+        if n > 1:
+            for a in range(0, n, tile_tokens):
+                tiles.append((s + min(n, a + tile_tokens), t + a, min(tile_tokens, n - a)))
+        t += n
+    tiles.sort(key=lambda x: -x[0])
+    host = torch.tensor([[f for _, f, _ in tiles], [c for _, _, c in tiles]], dtype=I32)
+    dev = host.to(device, non_blocking=True)
+    return dev[0], dev[1], len(tiles)
 
 
 # ------------------------------------------------------------------------------------- sampling

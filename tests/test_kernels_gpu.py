@@ -173,7 +173,10 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
 
 
 class _Batch:
-    pass
+    def prefill_tiles(self, tile_tokens):
+        from miniserve_amd.kernels.ops import build_prefill_tiles
+
+        return build_prefill_tiles(self.row_lens, self.row_starts_host, tile_tokens, DEV)
 
 
 def make_batch(lens_new, starts):
@@ -182,6 +185,7 @@ def make_batch(lens_new, starts):
     batch.token_row = torch.tensor([i for i, n in enumerate(lens_new) for _ in range(n)], dtype=torch.int32, device=DEV)
     batch.positions = torch.tensor([s + j for s, n in zip(starts, lens_new) for j in range(n)], dtype=torch.int32, device=DEV)
     batch.max_kv_len = max(s + n for s, n in zip(starts, lens_new))
+    batch.row_lens, batch.row_starts_host = list(lens_new), list(starts)
     n_dec = sum(1 for n in lens_new if n == 1)
     batch.num_decode_tokens = n_dec
     batch.decode_tokens = batch.prefill_tokens = None
@@ -279,6 +283,26 @@ def test_paged_attention(ops, dtype, hq, hkv, d, page, lens_new, starts, window)
 )
 def test_decode_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost):
     attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=30, boost=boost)
+
+
+@pytest.mark.parametrize(
+    "hq,hkv,d,lens_new,starts,window,boost",
+    [
+        (16, 8, 128, [200], [0], 0, (0, 5)),                          # a whole prompt, several tiles
+        (16, 8, 128, [64, 65, 2], [0, 0, 0], 0, None),                # a full tile, one token more, the shortest portion
+        (16, 8, 128, [70], [1000], 0, (0, 17)),                       # a portion deep into a sequence, a far key
+        (16, 8, 128, [33, 1, 90, 1], [31, 200, 64, 0], 0, (2, 63)),   # portions beside decode rows
+        (32, 8, 128, [50, 40], [10, 300], 0, (1, 299)),               # four heads per group: 32 tokens per tile
+        (64, 8, 128, [40], [100], 0, (0, 3)),                         # eight heads per group
+        (14, 2, 64, [100, 3], [0, 77], 0, (0, 50)),                   # seven heads per group: 18 tokens per tile, rows idle
+        (6, 6, 64, [150], [20], 0, None),                             # one head per group: 128 tokens per tile
+        (16, 8, 128, [150, 30], [0, 500], 40, (0, 149 - 39)),         # a window: its first key stands out
+        (16, 8, 128, [130], [300], 200, (0, 230)),                    # a window wider than the tile
+        (6, 6, 64, [300], [0], 17, None),                             # a window narrower than a key tile
+    ],
+)
+def test_prefill_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost):
+    attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=40, boost=boost)
 
 
 def test_decode_splits_rule(ops):
