@@ -40,6 +40,7 @@ def main() -> int:
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill measurement")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps eagerly")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -102,11 +103,14 @@ def main() -> int:
             eng.abort(r.rid)
         return dt, mean_ctx, eng
 
-    dt, mean_ctx, eng = decode_run(args.batch, args.steps, args.warmup)
+    if args.prefill_only:
+        dt, mean_ctx, eng = 1.0, 0.0, None
+    else:
+        dt, mean_ctx, eng = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     weight_bytes = model.decode_read_bytes()
-    kv_bytes = args.batch * mean_ctx * eng.runner.pool.bytes_per_token()
+    kv_bytes = args.batch * mean_ctx * (eng.runner.pool.bytes_per_token() if eng else 0)
     achieved = (weight_bytes + kv_bytes) / (dt / args.steps) / 1e9
     del eng
 
@@ -153,7 +157,7 @@ def main() -> int:
                           "frac": round(flops / pre / peak, 4)}
         del runner
         points = {}
-        for b, steps in ((1, 64), (64, 24)):
+        for b, steps in ((1, 64), (64, 24)) if not args.prefill_only else ():
             d, _, e = decode_run(b, steps, 8)
             points[f"decode_b{b}"] = round(b * steps / d, 1)
             del e

@@ -63,12 +63,23 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
 #pragma unroll
   for (int i = 0; i < DB; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // Page ids of a chunk are fetched one iteration ahead, so that their latency is not in the chain
+  // table -> page -> keys of every iteration.
+  int p0n = 0, p1n = 0;
+  if (c_begin + wave < c_end) {
+    const int t0 = lo_al + (c_begin + wave) * CHUNK;
+    p0n = table[t0 / PAGE];
+    p1n = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0n;
+  }
   for (int c = c_begin + wave; c < c_end; c += 4) {
     const int t0 = lo_al + c * CHUNK;
-    int p0 = table[t0 / PAGE];
-    int p1 = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0;
-    p0 = max(p0, 0);  // a page behind the window was given back: its tokens are masked below
-    p1 = max(p1, 0);
+    const int p0 = max(p0n, 0);  // a page behind the window was given back: its tokens are masked below
+    const int p1 = max(p1n, 0);
+    if (c + 4 < c_end) {
+      const int tn = t0 + 4 * CHUNK;
+      p0n = table[tn / PAGE];
+      p1n = (tn + PAGE < kv_len) ? table[tn / PAGE + 1] : p0n;
+    }
     const bf16* k0 = kc + (((size_t)p0 * Hkv + kvh) * PAGE + r) * D + g * 8;
     const bf16* k1 = kc + (((size_t)p1 * Hkv + kvh) * PAGE + r) * D + g * 8;
     bf16x8 ka[KK], kb[KK];

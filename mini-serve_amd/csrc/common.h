@@ -46,4 +46,18 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float* red
   return total;
 }
 
+// Sum of `splits` floats spaced `stride` apart, added in ascending order. Loads are issued eight at a
+// time so that they overlap; absent splits contribute an exact zero.
+__device__ __forceinline__ float sum_splits(const float* __restrict__ p, int splits, size_t stride) {
+  float acc = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (s0 + u < splits) ? p[(size_t)(s0 + u) * stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u];
+  }
+  return acc;
+}
+
 static inline int launch_status() { return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED; }

@@ -3,8 +3,8 @@
 //
 //  * tile kernel   (prefill, M large): BM x BN macro-tiles staged through LDS in K-slabs of 64 with a
 //                  register prefetch of the next slab; 4 waves in a 2 x 2 grid of wave tiles.
-//  * skinny kernel (decode, M <= 64): pure weight streaming. A wave owns 16 weight rows and walks
-//                  all of K with 32-byte loads per lane; the few activation rows come from LDS.
+//  * small-M kernel (decode, M <= 64): pure weight streaming. A wave owns 16 weight rows and a slice
+//                  of K, with 32-byte loads per lane; K is split over the grid into partial sums.
 //
 // Operand roles: the weight rows are the MFMA's A operand (its row index i = n) and the activation
 // rows the B operand (column index j = m), so a lane ends up with four consecutive n of one m and
@@ -13,7 +13,7 @@
 // Layout of v_mfma_f32_16x16x32_bf16 (lane l, g = l / 16, r = l % 16):
 //   A operand: 8 values A[i = r][k = 8 g .. 8 g + 7]     B operand: 8 values B[k = 8 g .. 8 g + 7][j = r]
 //   result:    4 values D[i = 4 g + 0..3][j = r]
-// Any permutation of k that is the same for both operands leaves the result unchanged; the skinny
+// Any permutation of k that is the same for both operands leaves the result unchanged; the small-M
 // kernel uses that to let a lane load 16 consecutive k at once.
 #include "common.h"
 
@@ -156,103 +156,86 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
 }
 
 // ---------------------------------------------------------------------------------------------
-// Skinny kernel: M <= 16 * MB rows of X. Block = 4 waves = 64 weight rows. K is walked in slabs of
-// KS; the X slab is staged in LDS once per block and shared by its waves.
-#define KS 256
-#define XS_STRIDE (KS + 8)
+// Small-M kernel: M <= 16 * MB rows of X (a decode step). Pure weight streaming: a wave owns 16 weight
+// rows and a slice of K; per step of 64 k each lane loads 32 bytes of its weight row and issues two
+// MFMAs per 16-row block of X. With MB == 1 the matching 32 bytes of an X row come straight from
+// global memory (X is a few KB and stays in the vector cache; no LDS, no barrier); with MB > 1 the
+// block's four waves stage the X slab of their common K slice in LDS. K is split over blockIdx.y so
+// that even a 1024-row matrix gives every CU several waves; each split writes float partial sums
+// P[split, M, N], which the caller's next kernel (or the reduction below) sums in ascending split
+// order. The number of splits depends on N and K alone, never on M: a row's result does not depend on
+// the batch it is in (within the same MB).
+#define SMALL_SLAB 256  // k per iteration: four steps of 64
+#define XS_STRIDE (SMALL_SLAB + 8)
 
 template <int MB>
-__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
-                                                               void* __restrict__ C, int mode, int M, int N, int K,
-                                                               int ldx, int ldc) {
-  __shared__ __attribute__((aligned(16))) bf16 xs[MB * 16 * XS_STRIDE];
+__global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                              float* __restrict__ P, int M, int N, int K, int ldx,
+                                                              int steps_per_split) {
+  __shared__ __attribute__((aligned(16))) bf16 xs[MB > 1 ? MB * 16 * XS_STRIDE : 8];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int nb = blockIdx.x * 64 + wave * 16;
+  const int nb = (blockIdx.x * 4 + wave) * 16;
   const int n = nb + r;
+  const int k_begin = blockIdx.y * steps_per_split * 64;
+  const int k_end = min(K, k_begin + steps_per_split * 64);
   const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
 
   floatx4 acc[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  for (int ks = 0; ks < K; ks += KS) {
-    __syncthreads();
-    // X slab [MB * 16][KS] into LDS, 16-byte chunks.
-    for (int c = tid; c < MB * 16 * (KS / 8); c += 256) {
-      const int m = c / (KS / 8), kc = (c % (KS / 8)) * 8;
-      const Chunk v = load_chunk(X, m, M, ks + kc, K, ldx, vecx);
-      *reinterpret_cast<uint4*>(&xs[m * XS_STRIDE + kc]) = v.u;
-    }
-    // This lane's weights of the slab: per block of 64 k, 16 consecutive k at offset 16 g.
-    Chunk w[KS / 64][2];
+  for (int k0 = k_begin; k0 < k_end; k0 += SMALL_SLAB) {
+    // This lane's weights of the slab: per step of 64 k, 16 consecutive k at offset 16 g. Chunks at or
+    // beyond k_end are asked for at K, where load_chunk yields zeros.
+    Chunk w[SMALL_SLAB / 64][2];
 #pragma unroll
-    for (int b = 0; b < KS / 64; ++b) {
-      const int k = ks + b * 64 + g * 16;
-      w[b][0] = load_chunk(W, n, N, k, K, K, vecw);
-      w[b][1] = load_chunk(W, n, N, k + 8, K, K, vecw);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int b = 0; b < KS / 64; ++b) {
-#pragma unroll
-      for (int i = 0; i < MB; ++i) {
-        const bf16* xp = &xs[(i * 16 + r) * XS_STRIDE + b * 64 + g * 16];
-        const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp);
-        const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + 8);
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[b][0].v, x0, acc[i], 0, 0, 0);
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[b][1].v, x1, acc[i], 0, 0, 0);
-      }
-    }
-  }
-  const bool vec_store = (ldc % 4 == 0);
-#pragma unroll
-  for (int i = 0; i < MB; ++i) store4(C, mode, i * 16 + r, nb + g * 4, M, N, ldc, acc[i], vec_store);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Small-M kernel: M <= 16 rows of X (a decode step of a small batch). No LDS, no barriers: a wave owns
-// 16 weight rows and a slice of K; per step of 64 k each lane loads 32 bytes of its weight row and
-// the matching 32 bytes of an X row (X is a few KB and stays in the vector cache), and issues two
-// MFMAs. K is split over blockIdx.y so that even a 1024-row matrix gives every CU several waves;
-// each split writes float partial sums P[split, M, N], summed afterwards in ascending split order.
-// The number of splits depends on N and K alone, never on M: a row's result does not depend on
-// the batch it is in.
-#define SMALL_UNROLL 4
-
-__global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
-                                                              float* __restrict__ P, int M, int N, int K, int ldx,
-                                                              int steps_per_split) {
-  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  const int r = lane % 16, g = lane / 16;
-  const int nb = (blockIdx.x * 4 + wave) * 16;
-  if (nb >= N) return;
-  const int n = nb + r;
-  const int k_begin = blockIdx.y * steps_per_split * 64;
-  const int k_end = min(K, k_begin + steps_per_split * 64);
-  const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
-
-  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = k_begin; k0 < k_end; k0 += 64 * SMALL_UNROLL) {
-    Chunk w[SMALL_UNROLL][2], x[SMALL_UNROLL][2];
-#pragma unroll
-    for (int u = 0; u < SMALL_UNROLL; ++u) {
-      const int k = k0 + u * 64 + g * 16;  // beyond k_end only where k_end == K: load_chunk zero-fills
+    for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+      const int k = k0 + u * 64 + g * 16;
       const int kw = k < k_end ? k : K;
       w[u][0] = load_chunk(W, n, N, kw, K, K, vecw);
       w[u][1] = load_chunk(W, n, N, kw + 8, K, K, vecw);
-      x[u][0] = load_chunk(X, r, M, kw, K, ldx, vecx);
-      x[u][1] = load_chunk(X, r, M, kw + 8, K, ldx, vecx);
     }
+    if (MB == 1) {
+      Chunk x[SMALL_SLAB / 64][2];
 #pragma unroll
-    for (int u = 0; u < SMALL_UNROLL; ++u) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, x[u][0].v, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, x[u][1].v, acc, 0, 0, 0);
+      for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+        const int k = k0 + u * 64 + g * 16;
+        const int kw = k < k_end ? k : K;
+        x[u][0] = load_chunk(X, r, M, kw, K, ldx, vecx);
+        x[u][1] = load_chunk(X, r, M, kw + 8, K, ldx, vecx);
+      }
+#pragma unroll
+      for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, x[u][0].v, acc[0], 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, x[u][1].v, acc[0], 0, 0, 0);
+      }
+    } else {
+      __syncthreads();  // the previous slab has been consumed
+      for (int c = tid; c < MB * 16 * (SMALL_SLAB / 8); c += 256) {
+        const int m = c / (SMALL_SLAB / 8), kc = (c % (SMALL_SLAB / 8)) * 8;
+        const int k = k0 + kc;
+        const Chunk v = load_chunk(X, m, M, k < k_end ? k : K, K, ldx, vecx);
+        *reinterpret_cast<uint4*>(&xs[m * XS_STRIDE + kc]) = v.u;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+          const bf16* xp = &xs[(i * 16 + r) * XS_STRIDE + u * 64 + g * 16];
+          const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp);
+          const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + 8);
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, x0, acc[i], 0, 0, 0);
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, x1, acc[i], 0, 0, 0);
+        }
+      }
     }
   }
-  // acc[i] = C[m = r][n = nb + 4 g + i]
+  // acc[i][e] = C[m = 16 i + r][n = nb + 4 g + e]
   float* dst = P + (size_t)blockIdx.y * M * N;
-  store4(dst, 1, r, nb + g * 4, M, N, N, acc, N % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < MB; ++i) store4(dst, 1, i * 16 + r, nb + g * 4, M, N, N, acc[i], N % 4 == 0);
 }
 
 // C (mode 0 bf16 / 1 float / 2 float +=) from the partial sums, in ascending split order.
@@ -260,38 +243,48 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ P, void* __restri
                                      int N, int ldc) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x, m = blockIdx.y;
   if (n >= N) return;
-  float v = 0.f;
-  for (int s = 0; s < splits; ++s) v += P[((size_t)s * M + m) * N + n];
+  const float v = sum_splits(P + (size_t)m * N + n, splits, (size_t)M * N);
   const size_t at = (size_t)m * ldc + n;
   if (mode == 0) ((bf16*)C)[at] = static_cast<bf16>(v);
   else if (mode == 1) ((float*)C)[at] = v;
   else ((float*)C)[at] += v;
 }
 
-// Splits of K for the small-M kernel: enough waves to fill the chip, at least two 64-k steps each.
+extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, int M, int N, int ldc, hipStream_t st) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (splits < 1 || ldc < N || mode < 0 || mode > 2 || M > 65535) return MS_BAD_ARG;
+  splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(P, C, mode, splits, M, N, ldc);
+  return launch_status();
+}
+
+// Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
+// its loads at once, unless that would make more than about 8192 waves (then longer slices).
 extern "C" int ms_gemm_bf16_small_splits(int N, int K) {
   const int steps = (K + 63) / 64;
   const int row_blocks = (N + 15) / 16;
-  int want = (1024 + row_blocks - 1) / row_blocks;
-  int most = steps / 2 > 0 ? steps / 2 : 1;
-  int s = want < most ? want : most;
-  if (s < 1) s = 1;
+  int s = (steps + 3) / 4;
+  const int most = 8192 / row_blocks > 0 ? 8192 / row_blocks : 1;
+  if (s > most) s = most;
   const int per = (steps + s - 1) / s;
   return (steps + per - 1) / per;  // no empty split
 }
 
-// X [M <= 16, K] * W [N, K]^T. `partials` holds splits * M * N floats (splits from
+// X [M <= 64, K] * W [N, K]^T. `partials` holds splits * M * N floats (splits from
 // ms_gemm_bf16_small_splits). With reduce != 0 the partial sums are folded into C here; otherwise the
 // caller's next kernel sums them.
 extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials, void* C, int mode, int reduce, int M,
                                   int N, int K, int ldx, int ldc, hipStream_t st) {
   if (M <= 0 || N <= 0) return MS_OK;
-  if (M > 16 || K <= 0 || ldx < K || partials == nullptr) return MS_BAD_ARG;
+  if (M > 64 || K <= 0 || ldx < K || partials == nullptr) return MS_BAD_ARG;
   const int splits = ms_gemm_bf16_small_splits(N, K);
   const int steps = (K + 63) / 64;
   const int per = (steps + splits - 1) / splits;
   dim3 grid((N + 63) / 64, splits);
-  gemm_bf16_small_kernel<<<grid, 256, 0, st>>>((const bf16*)X, (const bf16*)W, partials, M, N, K, ldx, per);
+  const bf16* x = (const bf16*)X;
+  const bf16* w = (const bf16*)W;
+  if (M <= 16) gemm_bf16_small_kernel<1><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
+  else if (M <= 32) gemm_bf16_small_kernel<2><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
+  else gemm_bf16_small_kernel<4><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
   if (reduce) {
     if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
     splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);
@@ -306,13 +299,6 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   if (K <= 0 || ldx < K || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
-  if (M <= 64) {
-    dim3 grid((N + 63) / 64);
-    if (M <= 16) gemm_bf16_skinny_kernel<1><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
-    else if (M <= 32) gemm_bf16_skinny_kernel<2><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
-    else gemm_bf16_skinny_kernel<4><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
-    return launch_status();
-  }
   // Large tiles when they still give every CU work; small tiles otherwise.
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
   if (big >= 256) {

@@ -22,15 +22,18 @@ _ERRORS = {1: "bad argument", 2: "unsupported size", 3: "kernel launch failed"}
 
 _SIGNATURES = {
     "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
-    "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
+    "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int, _c_ll, _c_void],
     "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
-    "ms_qk_norm_rope_store": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int,
-                              _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void,
+                              _c_int, _c_float, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_void],
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_small_splits": [_c_int, _c_int],
+    "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
@@ -93,6 +96,36 @@ def _ptr(t) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+class SplitSum:
+    """A matrix that exists only as partial sums: its value is ``parts.sum(0)`` (float32
+    ``[splits, M, N]``, to be added in ascending split order). The small-M matrix product leaves its
+    result in this form so that the kernel that consumes it does the summing and no kernel of its own
+    is spent on it. ``accumulate`` marks a sum that still has to be added to the residual stream."""
+
+    __slots__ = ("parts",)
+
+    def __init__(self, parts: torch.Tensor):
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return tuple(self.parts.shape[1:])
+
+    @property
+    def splits(self) -> int:
+        return self.parts.shape[0]
+
+    @property
+    def stride(self) -> int:
+        return self.parts.shape[1] * self.parts.shape[2]
+
+
+def _check_split(v: SplitSum, name: str, shape) -> None:
+    _dev(v.parts, name, F32, 3)
+    if v.shape != tuple(shape):
+        raise ValueError(f"{name} holds partial sums of a {v.shape} matrix, expected {tuple(shape)}")
+
+
 # ------------------------------------------------------------------------------------- elementwise
 
 
@@ -107,7 +140,11 @@ def embed(token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None) -> torch.Tensor:
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None,
+            add: SplitSum | None = None) -> torch.Tensor:
+    """RMSNorm of the float32 rows of ``x`` (all, or those named by ``rows``). ``add``: a pending sum that
+    is added to the rows first; without ``rows`` also into ``x`` itself (in place), with ``rows`` (which
+    may name a row twice) ``x`` is left unchanged."""
     _dev(x, "x", F32, 2)
     _dev(weight, "weight", (F32, BF16), 1)
     if weight.shape[0] != x.shape[1]:
@@ -118,16 +155,33 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: 
     if rows is not None:
         _dev(rows, "rows", I32, 1)
         n = rows.shape[0]
+    parts, splits, stride = None, 0, 0
+    if add is not None:
+        _check_split(add, "add", x.shape)
+        parts, splits, stride = add.parts.data_ptr(), add.splits, add.stride
     out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
     _check(library().ms_rmsnorm(x.data_ptr(), weight.data_ptr(), int(weight.dtype == BF16), out.data_ptr(),
-                                int(out_dtype == BF16), _ptr(rows), n, x.shape[1], float(eps), _stream()), "rmsnorm")
+                                int(out_dtype == BF16), _ptr(rows), n, x.shape[1], float(eps), parts, splits, stride,
+                                _stream()), "rmsnorm")
     return out
 
 
-def act_mul(gu: torch.Tensor, activation: str = "silu") -> torch.Tensor:
-    """``act(gu[:, :I]) * gu[:, I:]`` for ``gu [T, 2 I]``."""
+def act_mul(gu, activation: str = "silu", out_dtype=None) -> torch.Tensor:
+    """``act(gu[:, :I]) * gu[:, I:]`` for ``gu [T, 2 I]``, a tensor or a ``SplitSum`` (then ``out_dtype``
+    names the result's dtype)."""
     if activation != "silu":
         raise NotImplementedError(f"activation {activation!r}")
+    if isinstance(gu, SplitSum):
+        _dev(gu.parts, "gu", F32, 3)
+        t, width = gu.shape
+        if width % 2 or out_dtype not in (F32, BF16):
+            raise ValueError("gate/up partial sums need an even width and an output dtype")
+        out = torch.empty((t, width // 2), dtype=out_dtype, device=gu.parts.device)
+        for t0 in range(0, t, 32768):
+            n = min(32768, t - t0)
+            _check(library().ms_silu_mul_parts(gu.parts[:, t0:].data_ptr(), gu.splits, gu.stride, out[t0:].data_ptr(),
+                                               int(out_dtype == BF16), n, width // 2, _stream()), "silu_mul")
+        return out
     _dev(gu, "gu", (F32, BF16), 2)
     if gu.shape[1] % 2:
         raise ValueError("gate/up buffer needs an even width")
@@ -155,14 +209,19 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------------- matrix products
 
-SMALL_M = 16  # rows up to which the split-K weight-streaming kernel runs
+SMALL_M = 64  # rows up to which the split-K weight-streaming kernel runs
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None) -> torch.Tensor:
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None,
+           defer: bool = False):
     """``x [M, K] @ weight [N, K]^T``. Either returns a new ``[M, N]`` tensor of ``out_dtype``, or adds
-    the product into the float32 tensor ``accumulate_into`` (the residual stream) and returns it.
+    the product into the float32 tensor ``accumulate_into`` (the residual stream) and returns None.
     The weight's dtype picks the arithmetic: float32 weights run the true 32-bit kernel (``x`` is
-    widened first if needed), bfloat16 weights the matrix-core kernel with float32 accumulation."""
+    widened first if needed), bfloat16 weights the matrix-core kernels with float32 accumulation.
+
+    ``defer=True`` allows the result to come back as a ``SplitSum`` (partial sums that the consuming
+    kernel adds up) where the small-M kernel produced it in that form; with ``accumulate_into`` the
+    returned ``SplitSum`` is what still has to be added to that tensor."""
     _dev(x, "x", (F32, BF16), 2)
     _dev(weight, "weight", (F32, BF16), 2)
     m, k = x.shape
@@ -173,46 +232,77 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
         _dev(accumulate_into, "accumulate_into", F32, 2)
         if tuple(accumulate_into.shape) != (m, n):
             raise ValueError(f"linear: accumulator is {tuple(accumulate_into.shape)}, expected {(m, n)}")
-        out = accumulate_into
-    else:
-        if out_dtype not in (F32, BF16):
-            raise TypeError(f"unsupported output dtype {out_dtype}")
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    elif out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    lib = library()
+    if weight.dtype == BF16 and m <= SMALL_M:
+        xa = cast(x, BF16)
+        splits = lib.ms_gemm_bf16_small_splits(n, k)
+        if splits == 1 and accumulate_into is None and out_dtype == F32:
+            out = torch.empty((m, n), dtype=F32, device=x.device)  # the single partial sum is the result
+            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), None, 1, 0, m, n, k, k, n,
+                                          _stream()), "gemm_bf16_small")
+            return out
+        parts = torch.empty((splits, m, n), dtype=F32, device=x.device)
+        if defer:
+            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), None, 1, 0, m, n, k, k, n,
+                                          _stream()), "gemm_bf16_small")
+            return SplitSum(parts)
+        out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
+        mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
+        _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), out.data_ptr(), mode, 1, m, n, k,
+                                      k, n, _stream()), "gemm_bf16_small")
+        return None if accumulate_into is not None else out
+    out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
     if weight.dtype == F32:
         xa = cast(x, F32)
         mode = 1 if accumulate_into is not None else (0 if out.dtype == F32 else 2)
-        _check(library().ms_gemm_f32(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
-               "gemm_f32")
+        _check(lib.ms_gemm_f32(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()), "gemm_f32")
     else:
         xa = cast(x, BF16)
         mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
-        lib = library()
-        if m <= SMALL_M:
-            splits = lib.ms_gemm_bf16_small_splits(n, k)
-            if splits == 1 and mode == 1:
-                parts, reduce = out, 0  # the single partial sum is the result
-            else:
-                parts, reduce = torch.empty((splits, m, n), dtype=F32, device=x.device), 1
-            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), out.data_ptr(), mode, reduce,
-                                          m, n, k, k, n, _stream()), "gemm_bf16_small")
-        else:
-            _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()),
-                   "gemm_bf16")
-    return out
+        _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()), "gemm_bf16")
+    return None if accumulate_into is not None else out
+
+
+def add_pending(residual: torch.Tensor, pending: SplitSum | None) -> None:
+    """``residual += pending`` for callers whose next kernel cannot take a pending sum itself."""
+    if pending is None:
+        return
+    _dev(residual, "residual", F32, 2)
+    _check_split(pending, "pending", residual.shape)
+    m, n = residual.shape
+    _check(library().ms_splitk_reduce(pending.parts.data_ptr(), residual.data_ptr(), 2, pending.splits, m, n, n, _stream()),
+           "splitk_reduce")
 
 
 # ------------------------------------------------------------------------------------- attention
 
 
 def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq, rot_dim, k_cache, v_cache,
-                       num_heads, num_kv_heads, head_dim) -> None:
-    """In place on ``qkv [T, (Hq + 2 Hkv) D]``: per-head RMSNorm of q and k (if weights are given),
-    rotation by ``positions`` (if ``inv_freq`` is given), q written back, k and v stored into the
-    cache pages at ``slots`` (skipped when ``slots`` is None)."""
-    _dev(qkv, "qkv", (F32, BF16), 2)
-    t = qkv.shape[0]
-    if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
-        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {(num_heads + 2 * num_kv_heads) * head_dim}")
+                       num_heads, num_kv_heads, head_dim, out_dtype=None) -> torch.Tensor:
+    """From ``qkv [T, (Hq + 2 Hkv) D]`` (a tensor, or a ``SplitSum`` of it): per-head RMSNorm of q and k
+    (if weights are given), rotation by ``positions`` (if ``inv_freq`` is given), k and v stored into
+    the cache pages at ``slots`` (skipped when ``slots`` is None). Returns the tensor that holds the
+    finished queries in its first ``Hq * D`` columns: ``qkv`` itself (written in place), or for a
+    ``SplitSum`` a new ``[T, Hq D]`` tensor of ``out_dtype``."""
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    if isinstance(qkv, SplitSum):
+        _dev(qkv.parts, "qkv", F32, 3)
+        t = qkv.shape[0]
+        if qkv.shape[1] != width or out_dtype not in (F32, BF16):
+            raise ValueError(f"qkv partial sums have width {qkv.shape[1]}, expected {width}, and need an output dtype")
+        dtype = out_dtype
+        q_out = torch.empty((t, num_heads * head_dim), dtype=dtype, device=qkv.parts.device)
+        src, parts, splits, stride = None, qkv.parts.data_ptr(), qkv.splits, qkv.stride
+    else:
+        _dev(qkv, "qkv", (F32, BF16), 2)
+        t = qkv.shape[0]
+        if qkv.shape[1] != width:
+            raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
+        dtype = qkv.dtype
+        q_out = qkv
+        src, parts, splits, stride = qkv.data_ptr(), None, 0, 0
     _dev(positions, "positions", I32, 1)
     if positions.shape[0] != t:
         raise ValueError("one position per token is needed")
@@ -232,7 +322,7 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
         _dev(slots, "slots", I32, 1)
         if slots.shape[0] != t:
             raise ValueError("one slot per token is needed")
-        page_size = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
+        page_size = _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim)
     if inv_freq is not None:
         _dev(inv_freq, "inv_freq", F32, 1)
         if rot_dim % 2 or rot_dim > head_dim or inv_freq.shape[0] != rot_dim // 2:
@@ -240,10 +330,11 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
     else:
         rot_dim = 0
     _check(library().ms_qk_norm_rope_store(
-        qkv.data_ptr(), int(qkv.dtype == BF16), positions.data_ptr(), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
-        float(eps), _ptr(inv_freq), int(rot_dim), _ptr(k_cache) if slots is not None else None,
-        _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, page_size, _stream()),
-        "qk_norm_rope_store")
+        src, parts, splits, stride, q_out.data_ptr(), q_out.shape[1], int(dtype == BF16), positions.data_ptr(), _ptr(slots),
+        _ptr(q_weight), _ptr(k_weight), w_bf16, float(eps), _ptr(inv_freq), int(rot_dim),
+        _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, t, num_heads,
+        num_kv_heads, head_dim, page_size, _stream()), "qk_norm_rope_store")
+    return q_out
 
 
 def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
@@ -258,8 +349,8 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
     return page
 
 
-DECODE_TARGET_BLOCKS = 512  # workgroups the split decode kernel aims for
-DECODE_MIN_CHUNKS = 4  # 32-token chunks a split should at least hold
+DECODE_TARGET_BLOCKS = 1024  # workgroups the split decode kernel aims for
+DECODE_MIN_CHUNKS = 2  # 32-token chunks a split should at least hold
 
 
 def decode_splits(rows: int, num_kv_heads: int, max_kv_len: int) -> int:

@@ -6,7 +6,8 @@ of q and k, store of k and v into the cache, causal attention in which query hea
 head ``h // (heads / kv_heads)`` with ``scale`` on the scores, output projection. Here the three
 projections are one matrix product over row-concatenated weights (as the reference's fused path
 does, miniserve/model/fused.py:204-206); norm, rotation and cache store are one kernel; the output
-projection adds into the residual stream in its epilogue.
+projection adds into the residual stream in its epilogue, or (few rows) leaves partial sums pending
+for the next norm to add.
 
 ``window > 0`` restricts a query at position p to keys p-window+1 .. p (no counterpart in the
 reference). ``qk_norm_eps=None`` switches the per-head norms off; ``position`` may be ``none``.
@@ -69,21 +70,21 @@ class GQAttention(Mixer):
     def kv_need(self) -> KVNeed:
         return KVNeed(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, batch, cache, state, residual) -> None:
+    def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
-        qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype)
+        qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
         rot = self.position.rotation()
-        ops.qk_norm_rope_store(
+        q = ops.qk_norm_rope_store(
             qkv, batch.positions, cache.slots if cache.writes else None,
             self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps),
             rot.inv_freq if rot is not None else None, rot.dim if rot is not None else 0,
-            cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
+            cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, out_dtype=self.rt.dtype,
         )
         out = ops.paged_attention(
-            qkv, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
+            q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
             self.scale, self.window,
         )
-        ops.linear(out, self.o, accumulate_into=residual)
+        return ops.linear(out, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
         ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else [])

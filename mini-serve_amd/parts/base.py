@@ -4,17 +4,20 @@ A part is built from a ``PartSpec`` (its sizes and constants) and a ``Runtime`` 
 device, kernels); it declares the tensors it needs under its own prefix and receives exactly
 those. No part knows which model it is in. The kinds:
 
-* ``Norm``            ``forward(x_f32, rows=None) -> y``            (residual stream in, compute dtype out)
+* ``Norm``            ``forward(x_f32, rows=None, add=None) -> y``  (residual stream in, compute dtype out)
 * ``PositionEncoding`` ``rotation() -> Rotation | None``            (what a mixer's q/k are turned by)
-* ``Mixer``           ``forward(x, batch, cache, state, residual)`` (adds its output to ``residual``)
-* ``FeedForward``     ``forward(x, residual)``                      (adds its output to ``residual``)
-* ``Block``           ``forward(residual, batch, cache, state)``    (where norms and sums sit)
+* ``Mixer``           ``forward(x, batch, cache, state, residual) -> pending``
+* ``FeedForward``     ``forward(x, residual) -> pending``
+* ``Block``           ``forward(residual, batch, cache, state, pending) -> pending`` (where norms and sums sit)
 * ``Embedding``       ``forward(token_ids) -> residual``            (float32 ``[T, width]``)
 * ``Head``            ``forward(x) -> logits``                      (float32 ``[rows, vocab]``)
 
 The residual stream is float32 in every compute dtype: sums of layer outputs are never rounded
-to bfloat16. Mixers and feed-forwards add into it (so a matrix product can do the sum in its
-epilogue) instead of returning a tensor.
+to bfloat16. Mixers and feed-forwards do not return their output: they either add it into
+``residual`` themselves (a matrix product can do that in its epilogue) and return None, or return a
+*pending* sum (``ops.SplitSum``: partial sums that still have to be added to ``residual``). Whoever
+reads the residual stream next takes the pending sum along: a norm adds it while it normalises
+(``add=``), anything else calls ``ops.add_pending`` first.
 """
 
 from __future__ import annotations
@@ -97,7 +100,9 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, x, rows=None):
+    def forward(self, x, rows=None, add=None):
+        """Normalise rows of the float32 ``x`` plus ``add`` (a pending sum). Without ``rows``, ``x`` is
+        also brought up to date in place; with ``rows`` the stream is not read again and stays as it is."""
         raise NotImplementedError
 
 
@@ -113,12 +118,14 @@ class Mixer(Part):
     def state_need(self) -> StateNeed | None:
         return None
 
-    def forward(self, x, batch, cache, state, residual) -> None:
+    def forward(self, x, batch, cache, state, residual):
+        """Add the mixer's output to ``residual``, or return it as a pending sum."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, x, residual) -> None:
+    def forward(self, x, residual):
+        """Add the feed-forward's output to ``residual``, or return it as a pending sum."""
         raise NotImplementedError
 
 
@@ -128,7 +135,9 @@ class Block(Part):
         self.mixer = mixer
         self.feed_forward = feed_forward
 
-    def forward(self, residual, batch, cache, state) -> None:
+    def forward(self, residual, batch, cache, state, pending=None):
+        """Run the layer on ``residual`` (to which ``pending`` still has to be added); returns what is
+        pending afterwards."""
         raise NotImplementedError
 
 

@@ -29,9 +29,11 @@ class PreNormBlock(Block):
         self.mixer_norm.bind(tensors)
         self.ffn_norm.bind(tensors)
 
-    def forward(self, residual, batch, cache, state) -> None:
-        self.mixer.forward(self.mixer_norm.forward(residual), batch, cache, state, residual)
-        self.feed_forward.forward(self.ffn_norm.forward(residual), residual)
+    def forward(self, residual, batch, cache, state, pending=None):
+        x = self.mixer_norm.forward(residual, add=pending)
+        pending = self.mixer.forward(x, batch, cache, state, residual)
+        y = self.ffn_norm.forward(residual, add=pending)
+        return self.feed_forward.forward(y, residual)
 
     def parameters_bytes(self) -> int:
         return self.mixer_norm.parameters_bytes() + self.ffn_norm.parameters_bytes()

@@ -44,11 +44,11 @@ class GatedMLP(FeedForward):
         self.gate_up = torch.cat((g, u), dim=0).contiguous()
         self.down = tensors[p + "down_proj.weight"]
 
-    def forward(self, x, residual) -> None:
+    def forward(self, x, residual):
         ops = self.rt.ops
-        gu = ops.linear(x, self.gate_up, out_dtype=self.rt.dtype)
-        m = ops.act_mul(gu, self.activation)
-        ops.linear(m, self.down, accumulate_into=residual)
+        gu = ops.linear(x, self.gate_up, out_dtype=self.rt.dtype, defer=True)
+        m = ops.act_mul(gu, self.activation, out_dtype=self.rt.dtype)
+        return ops.linear(m, self.down, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.gate_up, self.down))

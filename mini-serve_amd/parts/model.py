@@ -95,13 +95,14 @@ class DecoderModel:
         """Run the batch's tokens through every run-order entry and return float32 logits
         ``[len(batch.want_rows), vocab]`` at the wanted flat token indices."""
         residual = self.embedding.forward(batch.token_ids)
+        pending = None  # a sum a layer left to be added to the residual stream by its next reader
         for e in self.spec.run_order:
             cache = pool.view(e.cache, batch, e.writes_cache) if e.cache is not None else None
             state = pool.state_view(e.cache, batch) if e.cache is not None else None
-            self.blocks[e.layer].forward(residual, batch, cache, state)
+            pending = self.blocks[e.layer].forward(residual, batch, cache, state, pending)
         if batch.num_wanted == 0:
             return None
-        x = self.final_norm.forward(residual, rows=batch.want_rows)
+        x = self.final_norm.forward(residual, rows=batch.want_rows, add=pending)
         return self.head.forward(x)
 
     def decode_read_bytes(self) -> int:

@@ -25,10 +25,11 @@ class RMSNorm(Norm):
     def bind(self, tensors) -> None:
         self.weight = tensors[self.spec["tensor"]]
 
-    def forward(self, x, rows=None):
+    def forward(self, x, rows=None, add=None):
         """``x``: float32 ``[T, width]``; ``rows``: optional int32 row indices to normalise (the
-        others are skipped). Returns the compute dtype, ``[T or len(rows), width]``."""
-        return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows)
+        others are skipped); ``add``: a pending sum added into the normalised rows of ``x`` first.
+        Returns the compute dtype, ``[T or len(rows), width]``."""
+        return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows, add)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

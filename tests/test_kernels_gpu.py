@@ -115,6 +115,46 @@ def test_gemm_bf16(ops, m, n, k):
     close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 40, 64])
+def test_pending_sums_feed_their_consumers(ops, m):
+    """The small-M product may leave partial sums for the next kernel to add: every consumer of such
+    a sum gives what it gives on the finished matrix."""
+    k, n = 1024, 1024
+    x, w = rand((m, k), BF16, 50), rand((n, k), BF16, 51, 0.05)
+    want = x.double() @ w.double().T
+    s = ops.linear(x, w, out_dtype=BF16, defer=True)
+    assert isinstance(s, ops.SplitSum) and s.splits > 1 and s.shape == (m, n)
+    close(s.parts.sum(0), want, 1e-5, "partial sums")
+    # the number of splits depends on the matrix alone, not on the rows
+    assert ops.linear(x[:1].contiguous(), w, out_dtype=BF16, defer=True).splits == s.splits
+    # residual stream: norm with the pending sum added first, rows or all
+    resid = rand((m, n), F32, 52)
+    nw = rand((n,), BF16, 53) + 1
+    full = resid.double() + want
+    normed = full / torch.sqrt((full * full).mean(-1, keepdim=True) + 1e-6) * nw.double()
+    r1 = resid.clone()
+    pend = ops.linear(x, w, accumulate_into=r1, defer=True)
+    assert isinstance(pend, ops.SplitSum) and torch.equal(r1, resid)  # nothing was added yet
+    close(ops.rmsnorm(r1, nw, 1e-6, BF16, add=pend), normed, 5e-3, "norm with pending sum")
+    close(r1, full, 1e-5, "residual brought up to date")
+    r2 = resid.clone()
+    rows = torch.tensor([m - 1, 0, 0], dtype=torch.int32, device=DEV)  # a row may be asked for twice
+    close(ops.rmsnorm(r2, nw, 1e-6, F32, rows, add=pend), normed[rows.long()], 1e-5, "norm of rows with pending sum")
+    assert torch.equal(r2, resid)  # with a row list the stream itself is left alone
+    r3 = resid.clone()
+    ops.add_pending(r3, pend)
+    close(r3, full, 1e-5, "add_pending")
+    # gated activation
+    gu = ops.linear(x, w, out_dtype=BF16, defer=True)
+    g, u = want[:, : n // 2], want[:, n // 2 :]
+    close(ops.act_mul(gu, out_dtype=BF16), g / (1 + torch.exp(-g)) * u, 6e-3, "act_mul of partial sums")
+    # without defer the same call returns the finished matrix / adds it
+    close(ops.linear(x, w, out_dtype=F32), want, 1e-5, "finished matrix")
+    r4 = resid.clone()
+    assert ops.linear(x, w, accumulate_into=r4) is None
+    close(r4, full, 1e-5, "accumulate")
+
+
 def test_linear_with_float32_weights_in_bfloat16_mode(ops):
     x, w = rand((9, 96), BF16, 14), rand((50, 96), F32, 15)
     close(ops.linear(x, w, out_dtype=BF16), x.double() @ w.double().T, 5e-3, "f32 weights, bf16 activations")
@@ -170,6 +210,13 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
     assert float((got_k[untouched.to(DEV)] - 7).abs().max()) == 0 and float((got_v[untouched.to(DEV)] - 7).abs().max()) == 0
     # position 0 is the identity of the rotation
     close(work.view(t, hq + 2 * hkv, d)[0, :hq], norm(q, qw)[0], tol, "position 0")
+    # the same from partial sums of qkv: queries come back in a tensor of their own
+    parts = torch.stack([qkv.float() * 0.25, qkv.float() * 0.5, qkv.float() * 0.25])
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = ops.qk_norm_rope_store(ops.SplitSum(parts), pos, slots, qw, kw, eps, inv_freq, rot, kc2, vc2, hq, hkv, d, out_dtype=dtype)
+    assert q2.shape == (t, hq * d)
+    close(q2.view(t, hq, d), qn, tol, "q from partial sums")
+    close(kc2.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)[sl], kn, tol, "k from partial sums")
 
 
 class _Batch:
@@ -306,8 +353,8 @@ def test_prefill_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost
 
 
 def test_decode_splits_rule(ops):
-    assert ops.decode_splits(1, 8, 4096) == 32 and ops.decode_splits(8, 8, 4096) == 8 and ops.decode_splits(64, 8, 4096) == 1
-    assert ops.decode_splits(1, 8, 100) == 1 and ops.decode_splits(1, 1, 40000) == 312 and ops.decode_splits(1, 8, 1) == 1
+    assert ops.decode_splits(1, 8, 4096) == 64 and ops.decode_splits(8, 8, 4096) == 16 and ops.decode_splits(64, 8, 4096) == 2
+    assert ops.decode_splits(1, 8, 100) == 2 and ops.decode_splits(1, 1, 40000) == 625 and ops.decode_splits(1, 8, 1) == 1
 
 
 def test_attention_one_token_returns_its_value(ops):
