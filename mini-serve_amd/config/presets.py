@@ -31,6 +31,18 @@ PRESETS: dict[str, dict] = {
         tie_word_embeddings=False, max_position_embeddings=512, sliding_window=24,
         layer_types=["sliding_attention", "full_attention", "sliding_attention", "sliding_attention"],
     ),
+    # Head sizes 64 and 128 with 16-token pages: the shapes the matrix-core attention kernels take.
+    "tinyD": _qwen3(
+        num_hidden_layers=2, hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+        intermediate_size=192, vocab_size=300, rope_theta=10000.0, rms_norm_eps=1e-6,
+        tie_word_embeddings=True, max_position_embeddings=2048,
+    ),
+    "tinyE": _qwen3(
+        num_hidden_layers=3, hidden_size=160, num_attention_heads=4, num_key_value_heads=1, head_dim=128,
+        intermediate_size=288, vocab_size=411, rope_theta=1e6, rms_norm_eps=1e-5,
+        tie_word_embeddings=False, max_position_embeddings=4096, sliding_window=100,
+        layer_types=["full_attention", "sliding_attention", "full_attention"],
+    ),
     "0.6B": _qwen3(
         num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
         intermediate_size=3072, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,

@@ -14,6 +14,8 @@ TINY = {
     "tinyA": (preset("tinyA"), 0, Init(0.02, None)),
     "tinyB": (preset("tinyB"), 1, Init(0.05, (0.5, 1.5))),
     "tinyC": (preset("tinyC"), 2, Init(0.04, (0.7, 1.3))),
+    "tinyD": (preset("tinyD"), 3, Init(0.03, (0.8, 1.2))),
+    "tinyE": (preset("tinyE"), 4, Init(0.04, (0.5, 1.5))),
 }
 
 

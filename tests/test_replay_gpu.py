@@ -17,7 +17,10 @@ from tolerances import check_logits
 pytestmark = pytest.mark.gpu
 
 DTYPES = ("float32", "bfloat16")
-LENGTHS = {"tinyA": [40, 7, 33, 64, 19, 90], "tinyB": [97, 3, 50, 65, 128, 31, 80], "tinyC": [100, 30, 77, 129, 48]}
+LENGTHS = {
+    "tinyA": [40, 7, 33, 64, 19, 90], "tinyB": [97, 3, 50, 65, 128, 31, 80], "tinyC": [100, 30, 77, 129, 48],
+    "tinyD": [300, 1, 65, 130, 2, 47], "tinyE": [520, 33, 257, 64, 150],
+}
 
 
 @pytest.fixture(scope="module")
@@ -132,4 +135,19 @@ def test_mixed_with_page_reuse(name, dtype, folders, truth, tmp_path):
             for i, s, n in entries:
                 check_logits(got[at : at + n], want[i][s : s + n], dtype, f"{name} request {i} tokens {s}..{s + n}")
                 at += n
+        assert rp.close() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(TINY))
+def test_first_tokens_one_by_one(name, dtype, folders, truth, tmp_path):
+    """A sequence fed one token at a time from its very first token: positions 0, 1, 2, ... on the
+    decode path, four sequences side by side."""
+    reqs, want = truth[name]
+    picked = [i for i in range(len(reqs)) if len(reqs[i]) >= 20][:4]
+    with Replay(folders[name], dtype, tmp_path / "out", 64 * len(picked)) as rp:
+        for p in range(20):
+            got = rp.step([(f"r{i}", [reqs[i][p]], [0]) for i in picked], end=[f"r{i}" for i in picked] if p == 19 else [])
+            for k, i in enumerate(picked):
+                check_logits(got[k : k + 1], want[i][p : p + 1], dtype, f"{name} request {i} position {p}")
         assert rp.close() == 0
