@@ -16,14 +16,55 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;  // 16 bytes in flight
 
 #define PAGE 16
 #define TK 64      // keys per tile
 #define ROWS 128   // query rows per block
 #define NQ 2       // 16-row blocks per wave
 
+// 16-byte chunks of a tile of TK keys: K [TK tokens][D] and V^T [D][TK tokens], spread over 256 threads.
 template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__device__ __forceinline__ void fetch_tile(u32x4 (&kreg)[TK * (D / 8) / 256], u32x4 (&vreg)[(TK / PAGE) * D * 2 / 256],
+                                           const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                           const int* __restrict__ table, int t0, int last_pos, int Hkv, int kvh, int tid) {
+#pragma unroll
+  for (int i = 0; i < TK * (D / 8) / 256; ++i) {
+    const int c = tid + i * 256;
+    const int tok = c / (D / 8), dc = c % (D / 8);
+    const int t = min(t0 + tok, last_pos);
+    const int page = max(table[t / PAGE], 0);  // a page behind the window was given back: masked later
+    kreg[i] = *reinterpret_cast<const u32x4*>(kc + (((size_t)page * Hkv + kvh) * PAGE + t % PAGE) * D + dc * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < (TK / PAGE) * D * 2 / 256; ++i) {
+    const int c = tid + i * 256;
+    const int pi = c / (2 * D), rem = c % (2 * D), d = rem / 2, half = rem % 2;
+    const int t = min(t0 + pi * PAGE, last_pos);
+    const int page = max(table[t / PAGE], 0);
+    vreg[i] = *reinterpret_cast<const u32x4*>(vc + (((size_t)page * Hkv + kvh) * D + d) * PAGE + half * 8);
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void stash_tile(const u32x4 (&kreg)[TK * (D / 8) / 256],
+                                           const u32x4 (&vreg)[(TK / PAGE) * D * 2 / 256], bf16* ks, bf16* vs, int tid) {
+  constexpr int KS = D + 8, VS = TK + 8;
+#pragma unroll
+  for (int i = 0; i < TK * (D / 8) / 256; ++i) {
+    const int c = tid + i * 256;
+    *reinterpret_cast<u32x4*>(&ks[(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = kreg[i];
+  }
+#pragma unroll
+  for (int i = 0; i < (TK / PAGE) * D * 2 / 256; ++i) {
+    const int c = tid + i * 256;
+    const int pi = c / (2 * D), rem = c % (2 * D);
+    *reinterpret_cast<u32x4*>(&vs[(rem / 2) * VS + pi * PAGE + (rem % 2) * 8]) = vreg[i];
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos,
@@ -82,25 +123,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int i = 0; i < DB; ++i) o[b][i] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int t0 = (kv_lo / TK) * TK; t0 <= last_pos; t0 += TK) {
+  // Global -> registers -> LDS, one tile ahead: the loads of tile i + 1 are in flight while tile i is
+  // being multiplied. (A fetch past the last tile reads clamped, valid addresses and is dropped.)
+  u32x4 kreg[TK * (D / 8) / 256], vreg[(TK / PAGE) * D * 2 / 256];
+  const float scale2 = scale * 1.44269504088896340736f;  // scores in units of log2: exp2 is one instruction
+  const int t_first = (kv_lo / TK) * TK;
+  fetch_tile<D>(kreg, vreg, kc, vc, table, t_first, last_pos, Hkv, kvh, tid);
+  for (int t0 = t_first; t0 <= last_pos; t0 += TK) {
     __syncthreads();  // the previous tile has been consumed
-    // K tile: 64 tokens x D, 16-byte chunks.
-    for (int c = tid; c < TK * (D / 8); c += 256) {
-      const int tok = c / (D / 8), dc = c % (D / 8);
-      const int t = min(t0 + tok, last_pos);
-      const int page = max(table[t / PAGE], 0);
-      const uint4 v = *reinterpret_cast<const uint4*>(kc + (((size_t)page * Hkv + kvh) * PAGE + t % PAGE) * D + dc * 8);
-      *reinterpret_cast<uint4*>(&ks[tok * KS + dc * 8]) = v;
-    }
-    // V^T tile: D x 64 tokens: per page and head element two 16-byte halves.
-    for (int c = tid; c < (TK / PAGE) * D * 2; c += 256) {
-      const int pi = c / (2 * D), rem = c % (2 * D), d = rem / 2, half = rem % 2;
-      const int t = min(t0 + pi * PAGE, last_pos);
-      const int page = max(table[t / PAGE], 0);
-      const uint4 v = *reinterpret_cast<const uint4*>(vc + (((size_t)page * Hkv + kvh) * D + d) * PAGE + half * 8);
-      *reinterpret_cast<uint4*>(&vs[d * VS + pi * PAGE + half * 8]) = v;
-    }
+    stash_tile<D>(kreg, vreg, ks, vs, tid);
     __syncthreads();
+    fetch_tile<D>(kreg, vreg, kc, vc, table, t0 + TK, last_pos, Hkv, kvh, tid);
     if (!wave_has_rows || t0 > wave_last_pos) continue;
     if (window > 0 && t0 + TK - 1 < wave_first_pos - window + 1) continue;
 
@@ -120,6 +153,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     }
     bf16x8 pf[NQ][TK / 32];
     float cq[NQ][4];
+    // A tile needs masks only where it crosses the diagonal or the window's edge for some row of the wave.
+    const bool masked = t0 + TK - 1 > wave_first_pos || (window > 0 && t0 <= wave_last_pos - window);
 #pragma unroll
     for (int b = 0; b < NQ; ++b) {
       // Scores of row r of block b: tokens t0 + tb * 16 + 4 g + i.
@@ -128,9 +163,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       for (int tb = 0; tb < TK / 16; ++tb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int t = t0 + tb * 16 + 4 * g + i;
-          const bool seen = !row_ok[b] || (t <= row_pos[b] && (window == 0 || t > row_pos[b] - window));
-          const float v = seen ? s[b][tb][i] * scale : -INFINITY;
+          float v = s[b][tb][i] * scale2;
+          if (masked) {
+            const int t = t0 + tb * 16 + 4 * g + i;
+            const bool seen = !row_ok[b] || (t <= row_pos[b] && (window == 0 || t > row_pos[b] - window));
+            v = seen ? v : -INFINITY;
+          }
           s[b][tb][i] = v;
           m_new = fmaxf(m_new, v);
         }
@@ -142,13 +180,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       for (int tb = 0; tb < TK / 16; ++tb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = expf(s[b][tb][i] - m_safe);
+          const float p = __builtin_amdgcn_exp2f(s[b][tb][i] - m_safe);
           psum += p;
           pf[b][tb / 2][(tb % 2) * 4 + i] = static_cast<bf16>(p);
         }
       psum += __shfl_xor(psum, 16, WAVE);
       psum += __shfl_xor(psum, 32, WAVE);
-      const float corr = expf(m_run[b] - m_safe);
+      const float corr = __builtin_amdgcn_exp2f(m_run[b] - m_safe);
       l_run[b] = l_run[b] * corr + psum;
       m_run[b] = m_new;
 #pragma unroll

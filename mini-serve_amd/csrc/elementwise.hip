@@ -161,89 +161,100 @@ extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf1
 }
 
 // ---------------------------------------------------------------------------------------------
-// One wave per (token, head slot). Head slots [0, Hq) are query heads, [Hq, Hq+Hkv) key heads,
-// [Hq+Hkv, Hq+2Hkv) value heads of the token's row in qkv [tokens, (Hq + 2 Hkv) * D].
+// One block of 4 waves per token; its waves take the token's head slots in turn. Head slots [0, Hq)
+// are query heads, [Hq, Hq+Hkv) key heads, [Hq+Hkv, Hq+2Hkv) value heads of the token's row in
+// qkv [tokens, (Hq + 2 Hkv) * D].
 //   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
-//         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j];
-//   q is written back in place; k and v go to the cache page of the token's slot
+//         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j] (sine and cosine are formed once per
+//         token and shared by all its heads);
+//   q goes to q_out; k and v go to the cache page of the token's slot
 //   (slot = page * page_size + offset; keys [pages, Hkv, page_size, D], values transposed within
 //   the page, [pages, Hkv, D, page_size]).
 // With slots == nullptr only the query heads are processed (the entry reads another entry's cache).
 #define MAX_HEAD_DIM 256
 template <typename T, typename TW>
-__global__ void qk_norm_rope_store_kernel(const T* qkv, const float* __restrict__ parts, int splits,
-                                          size_t split_stride, T* q_out, int q_out_stride,
-                                          const int* __restrict__ pos, const int* __restrict__ slots,
-                                          const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
-                                          const float* __restrict__ inv_freq, int rot, T* __restrict__ kc,
-                                          T* __restrict__ vc, int Hq, int Hkv, int D, int page_size) {
-  __shared__ float buf[MAX_HEAD_DIM];
-  const int t = blockIdx.x, hs = blockIdx.y, lane = threadIdx.x;
-  const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);
-  const size_t at = ((size_t)t * (Hq + 2 * Hkv) + hs) * D;
+__global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
+    const T* qkv, const float* __restrict__ parts, int splits, size_t split_stride, T* q_out, int q_out_stride,
+    const int* __restrict__ pos, const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw,
+    float eps, const float* __restrict__ inv_freq, int rot, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D,
+    int page_size, int heads) {
+  __shared__ float cs[MAX_HEAD_DIM / 2], sn[MAX_HEAD_DIM / 2];
+  __shared__ float buf[4][MAX_HEAD_DIM];
+  const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int half = rot / 2;
+  if (threadIdx.x < half) {
+    float s, c;
+    sincosf((float)pos[t] * inv_freq[threadIdx.x], &s, &c);
+    cs[threadIdx.x] = c;
+    sn[threadIdx.x] = s;
+  }
+  __syncthreads();
   constexpr int PER = MAX_HEAD_DIM / WAVE;
-  float x[PER];
-  float ss = 0.f;
+  for (int hs = wave; hs < heads; hs += 4) {
+    const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);
+    const size_t at = ((size_t)t * (Hq + 2 * Hkv) + hs) * D;
+    float x[PER];
+    float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int e = lane + i * WAVE;
-    float v = 0.f;
-    if (e < D) {
-      if (parts != nullptr) {
-        v = sum_splits(parts + at + e, splits, split_stride);
-      } else {
-        v = to_f32(qkv[at + e]);
-      }
-    }
-    x[i] = v;
-    ss += v * v;
-  }
-  T* dst = q_out + (size_t)t * q_out_stride + (size_t)hs * D;  // for a query head
-  size_t dst_step = 1;  // distance between consecutive head elements at the destination
-  if (kind == 1) {
-    const int s = slots[t];
-    dst = kc + (((size_t)(s / page_size) * Hkv + (hs - Hq)) * page_size + (s % page_size)) * D;
-  } else if (kind == 2) {
-    const int s = slots[t];
-    dst = vc + ((size_t)(s / page_size) * Hkv + (hs - Hq - Hkv)) * D * page_size + (s % page_size);
-    dst_step = page_size;
-  }
-  if (kind != 2) {
-    const TW* w = kind == 0 ? qw : kw;
-    if (w != nullptr) {
-      ss = wave_sum(ss);
-      const float rstd = rsqrtf(ss / (float)D + eps);
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int e = lane + i * WAVE;
-        if (e < D) x[i] = x[i] * rstd * to_f32(w[e]);
-      }
-    }
-    if (rot > 0) {
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int e = lane + i * WAVE;
-        if (e < D) buf[e] = x[i];
-      }
-      __syncthreads();
-      const int half = rot / 2;
-      const float p = (float)pos[t];
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int e = lane + i * WAVE;
-        if (e < rot) {
-          const int j = e < half ? e : e - half;
-          float sn, cs;
-          sincosf(p * inv_freq[j], &sn, &cs);
-          x[i] = e < half ? x[i] * cs - buf[e + half] * sn : x[i] * cs + buf[e - half] * sn;
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane + i * WAVE;
+      float v = 0.f;
+      if (e < D) {
+        if (parts != nullptr) {
+          v = sum_splits(parts + at + e, splits, split_stride);
+        } else {
+          v = to_f32(qkv[at + e]);
         }
       }
+      x[i] = v;
+      ss += v * v;
     }
-  }
+    T* dst = q_out + (size_t)t * q_out_stride + (size_t)hs * D;  // for a query head
+    size_t dst_step = 1;  // distance between consecutive head elements at the destination
+    if (kind == 1) {
+      const int s = slots[t];
+      dst = kc + (((size_t)(s / page_size) * Hkv + (hs - Hq)) * page_size + (s % page_size)) * D;
+    } else if (kind == 2) {
+      const int s = slots[t];
+      dst = vc + ((size_t)(s / page_size) * Hkv + (hs - Hq - Hkv)) * D * page_size + (s % page_size);
+      dst_step = page_size;
+    }
+    if (kind != 2) {
+      const TW* w = kind == 0 ? qw : kw;
+      if (w != nullptr) {
+        ss = wave_sum(ss);
+        const float rstd = rsqrtf(ss / (float)D + eps);
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int e = lane + i * WAVE;
-    if (e < D) dst[(size_t)e * dst_step] = from_f32<T>(x[i]);
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e < D) x[i] = x[i] * rstd * to_f32(w[e]);
+        }
+      }
+      if (rot > 0) {
+        // The wave exchanges the partners of its pairs through its own LDS row; a wave runs in
+        // lockstep, so no block barrier is needed between its write and its read.
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e < D) buf[wave][e] = x[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e < rot) {
+            const int j = e < half ? e : e - half;
+            x[i] = e < half ? x[i] * cs[j] - buf[wave][e + half] * sn[j] : x[i] * cs[j] + buf[wave][e - half] * sn[j];
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane + i * WAVE;
+      if (e < D) dst[(size_t)e * dst_step] = from_f32<T>(x[i]);
+    }
   }
 }
 
@@ -260,12 +271,10 @@ extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int sp
   if ((qw == nullptr) != (kw == nullptr)) return MS_BAD_ARG;
   if (rot > 0 && inv_freq == nullptr) return MS_BAD_ARG;
   const int heads = slots ? Hq + 2 * Hkv : Hq;
-  if (heads > 65535) return MS_BAD_ARG;
-  dim3 grid(tokens, heads);
-#define LAUNCH(T, TW)                                                                                                  \
-  qk_norm_rope_store_kernel<T, TW><<<grid, WAVE, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, \
-                                                           q_out_stride, pos, slots, (const TW*)qw, (const TW*)kw, eps,  \
-                                                           inv_freq, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size)
+#define LAUNCH(T, TW)                                                                                                   \
+  qk_norm_rope_store_kernel<T, TW><<<tokens, 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, \
+                                                            q_out_stride, pos, slots, (const TW*)qw, (const TW*)kw, eps,  \
+                                                            inv_freq, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
   if (is_bf16 && w_is_bf16) LAUNCH(bf16, bf16);
   else if (is_bf16) LAUNCH(bf16, float);
   else if (w_is_bf16) LAUNCH(float, bf16);

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
     for (int j = 0; j < FM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   Chunk xr[XCH], wr[WCH];
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       const int c = tid + i * 256;
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
       wr[i] = load_chunk(W, n0 + c / (BK / 8), N, k0 + (c % (BK / 8)) * 8, K, K, vecw);
     }
   };
-  auto stash = [&]() {
+  auto stash = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       const int c = tid + i * 256;
