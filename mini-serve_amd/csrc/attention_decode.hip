@@ -186,7 +186,8 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
   }
 }
 
-// Reduction of the splits in ascending order: grid (rows, Hq), D threads.
+// Reduction of the splits in ascending order: grid (rows, Hq), D threads. Loads go out eight splits
+// at a time so that their latencies overlap.
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
@@ -195,14 +196,29 @@ __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __re
   const int b = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const size_t base = ((size_t)b * Hq + head) * splits;
   float M = -INFINITY;
-  for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float m[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) m[u] = s0 + u < splits ? part_ml[(base + s0 + u) * 2] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) M = fmaxf(M, m[u]);
+  }
   float L = 0.f, O = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float m = part_ml[(base + s) * 2];
-    if (m == -INFINITY) continue;  // an empty split
-    const float f = expf(m - M);
-    L += part_ml[(base + s) * 2 + 1] * f;
-    O += part_o[(base + s) * D + d] * f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float m[8], l[8], o[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const bool in = s0 + u < splits;
+      m[u] = in ? part_ml[(base + s0 + u) * 2] : -INFINITY;
+      l[u] = in ? part_ml[(base + s0 + u) * 2 + 1] : 0.f;
+      o[u] = in ? part_o[(base + s0 + u) * D + d] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float f = m[u] == -INFINITY ? 0.f : expf(m[u] - M);  // an empty or absent split adds nothing
+      L += l[u] * f;
+      O += o[u] * f;
+    }
   }
   const int tok = tokens ? tokens[b] : b;
   out[((size_t)tok * Hq + head) * D + d] = static_cast<bf16>(O / L);

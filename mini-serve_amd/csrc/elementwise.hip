@@ -161,12 +161,12 @@ extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf1
 }
 
 // ---------------------------------------------------------------------------------------------
-// One block of 4 waves per token; its waves take the token's head slots in turn. Head slots [0, Hq)
+// One block of 4 waves per (token, four head slots): a wave per head slot. Head slots [0, Hq)
 // are query heads, [Hq, Hq+Hkv) key heads, [Hq+Hkv, Hq+2Hkv) value heads of the token's row in
 // qkv [tokens, (Hq + 2 Hkv) * D].
 //   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
 //         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j] (sine and cosine are formed once per
-//         token and shared by all its heads);
+//         block and shared by its four heads);
 //   q goes to q_out; k and v go to the cache page of the token's slot
 //   (slot = page * page_size + offset; keys [pages, Hkv, page_size, D], values transposed within
 //   the page, [pages, Hkv, D, page_size]).
@@ -181,6 +181,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   __shared__ float cs[MAX_HEAD_DIM / 2], sn[MAX_HEAD_DIM / 2];
   __shared__ float buf[4][MAX_HEAD_DIM];
   const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int hs = blockIdx.y * 4 + wave;  // this wave's head slot
   const int half = rot / 2;
   if (threadIdx.x < half) {
     float s, c;
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   }
   __syncthreads();
   constexpr int PER = MAX_HEAD_DIM / WAVE;
-  for (int hs = wave; hs < heads; hs += 4) {
+  if (hs < heads) {
     const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);
     const size_t at = ((size_t)t * (Hq + 2 * Hkv) + hs) * D;
     float x[PER];
@@ -271,8 +272,9 @@ extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int sp
   if ((qw == nullptr) != (kw == nullptr)) return MS_BAD_ARG;
   if (rot > 0 && inv_freq == nullptr) return MS_BAD_ARG;
   const int heads = slots ? Hq + 2 * Hkv : Hq;
+  if ((heads + 3) / 4 > 65535) return MS_BAD_ARG;
 #define LAUNCH(T, TW)                                                                                                   \
-  qk_norm_rope_store_kernel<T, TW><<<tokens, 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, \
+  qk_norm_rope_store_kernel<T, TW><<<dim3(tokens, (heads + 3) / 4), 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, \
                                                             q_out_stride, pos, slots, (const TW*)qw, (const TW*)kw, eps,  \
                                                             inv_freq, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
   if (is_bf16 && w_is_bf16) LAUNCH(bf16, bf16);
