@@ -20,8 +20,6 @@ typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;  
 
 #define PAGE 16
 #define TK 64      // keys per tile
-#define ROWS 128   // query rows per block
-#define NQ 2       // 16-row blocks per wave
 
 // 16-byte chunks of a tile of TK keys: K [TK tokens][D] and V^T [D][TK tokens], spread over 256 threads.
 template <int D>
@@ -63,13 +61,15 @@ __device__ __forceinline__ void stash_tile(const u32x4 (&kreg)[TK * (D / 8) / 25
   }
 }
 
-template <int D>
+template <int D, int NQ>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos,
     bf16* __restrict__ out, int Hq, int Hkv, float scale, int window) {
   constexpr int KK = D / 32, DB = D / 16;
+  constexpr int ROWS = 64 * NQ;  // query rows per block: 16 NQ per wave
+  constexpr int WROWS = 16 * NQ;
   constexpr int KS = D + 8;    // LDS row stride of the K tile (bf16)
   constexpr int VS = TK + 8;   // LDS row stride of the V^T tile
   __shared__ __attribute__((aligned(16))) bf16 ks[TK * KS];
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   bf16x8 qf[NQ][KK];
 #pragma unroll
   for (int b = 0; b < NQ; ++b) {
-    const int row = wave * 32 + b * 16 + r;
+    const int row = wave * WROWS + b * 16 + r;
     row_tok[b] = row / G;
     row_ok[b] = row_tok[b] < count && row < (ROWS / G) * G;
     row_pos[b] = pos0 + row_tok[b];
@@ -107,8 +107,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
   }
   // Highest position among this wave's rows: tiles beyond it hold nothing the wave may see.
-  const int wave_first_tok = (wave * 32) / G;
-  const int wave_last_tok = min(count - 1, (wave * 32 + 31) / G);
+  const int wave_first_tok = (wave * WROWS) / G;
+  const int wave_last_tok = min(count - 1, (wave * WROWS + WROWS - 1) / G);
   const bool wave_has_rows = wave_first_tok < count;
   const int wave_last_pos = pos0 + wave_last_tok;
   const int wave_first_pos = pos0 + wave_first_tok;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float inv_i = __shfl(inv, 4 * g + i, WAVE);
-      const int row = wave * 32 + b * 16 + 4 * g + i;
+      const int row = wave * WROWS + b * 16 + 4 * g + i;
       const int tok = row / G;
       if (tok < count && row < (ROWS / G) * G) {
         bf16* dst = out + ((size_t)(first + tok) * Hq + kvh * G + row % G) * D;
@@ -233,25 +233,29 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   }
 }
 
-// Tokens per tile for a group of G query heads per KV head.
-extern "C" int ms_attention_prefill_tile_tokens(int G) { return G >= 1 && G <= ROWS ? ROWS / G : 0; }
+// Query rows per block: 128 (two 16-row blocks per wave) when that still gives every CU two blocks,
+// else 64. Tokens per tile = rows / G.
+extern "C" int ms_attention_prefill_tile_tokens(int G, int rows) { return G >= 1 && G <= rows ? rows / G : 0; }
 
 extern "C" int ms_attention_prefill_bf16(const void* q, int q_stride, const void* kc, const void* vc,
                                          const int* block_table, int table_width, const int* tile_first,
-                                         const int* tile_count, int tiles, const int* token_row, const int* pos,
-                                         void* out, int Hq, int Hkv, int D, int page_size, float scale, int window,
-                                         hipStream_t st) {
+                                         const int* tile_count, int tiles, int rows_per_tile, const int* token_row,
+                                         const int* pos, void* out, int Hq, int Hkv, int D, int page_size, float scale,
+                                         int window, hipStream_t st) {
   if (tiles <= 0) return MS_OK;
   if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
-  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > ROWS || window < 0 || table_width <= 0 || q_stride < Hq * D ||
-      q_stride % 8 || (long long)tiles * Hkv > 2147483647LL)
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 64 || window < 0 || table_width <= 0 || q_stride < Hq * D ||
+      q_stride % 8 || (long long)tiles * Hkv > 2147483647LL || (rows_per_tile != 64 && rows_per_tile != 128))
     return MS_BAD_ARG;
   const unsigned grid = (unsigned)tiles * Hkv;
-#define LAUNCH(DD)                                                                                                    \
-  attn_prefill_kernel<DD><<<grid, 256, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, \
-                                                table_width, tile_first, tile_count, token_row, pos, (bf16*)out, Hq, Hkv, \
-                                                scale, window)
-  if (D == 128) LAUNCH(128); else LAUNCH(64);
+#define LAUNCH(DD, NN)                                                                                                  \
+  attn_prefill_kernel<DD, NN><<<grid, 256, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc,         \
+                                                    block_table, table_width, tile_first, tile_count, token_row, pos,   \
+                                                    (bf16*)out, Hq, Hkv, scale, window)
+  if (D == 128 && rows_per_tile == 128) LAUNCH(128, 2);
+  else if (D == 128) LAUNCH(128, 1);
+  else if (rows_per_tile == 128) LAUNCH(64, 2);
+  else LAUNCH(64, 1);
 #undef LAUNCH
   return launch_status();
 }

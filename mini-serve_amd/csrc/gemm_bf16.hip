@@ -71,10 +71,12 @@ __device__ __forceinline__ void store4(void* __restrict__ C, int mode, int m, in
 #define BK 64
 #define LDS_STRIDE (BK + 8)  // bf16 elements per LDS row: 144 bytes, keeps 16-byte alignment
 
+// blockIdx.z splits K into slices of k_per (a multiple of BK); slice z writes to C + z * c_split_stride
+// elements (float partial sums, mode 1), so that matrices with few output tiles still fill the chip.
 template <int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
-                                                             void* __restrict__ C, int mode, int M, int N, int K,
-                                                             int ldx, int ldc) {
+__global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                                void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
+                                                                int ldx, int ldc, int k_per, size_t c_split_stride) {
   constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
   constexpr int FM = WM / 16, FN = WN / 16;    // 16 x 16 fragments per wave tile
   constexpr int XCH = BM * (BK / 8) / 256;     // 16-byte chunks per thread per slab
@@ -86,7 +88,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
   const int r = lane % 16, g = lane / 16;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
-  const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
+  const bool vecx = (Kfull % 8 == 0) && (ldx % 8 == 0), vecw = (Kfull % 8 == 0);
+  const int k_lo = blockIdx.z * k_per;
+  const int K = min(Kfull, k_lo + k_per);  // this slice ends here; chunks beyond it read as zeros
+  void* C = mode == 1 ? (void*)((float*)Cbase + blockIdx.z * c_split_stride) : Cbase;
 
   floatx4 acc[FN][FM];
 #pragma unroll
@@ -104,7 +109,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
 #pragma unroll
     for (int i = 0; i < WCH; ++i) {
       const int c = tid + i * 256;
-      wr[i] = load_chunk(W, n0 + c / (BK / 8), N, k0 + (c % (BK / 8)) * 8, K, K, vecw);
+      wr[i] = load_chunk(W, n0 + c / (BK / 8), N, k0 + (c % (BK / 8)) * 8, K, Kfull, vecw);
     }
   };
   auto stash = [&]() __attribute__((always_inline)) {
@@ -120,10 +125,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(const bf16* __restr
     }
   };
 
-  fetch(0);
+  fetch(k_lo);
   stash();
   __syncthreads();
-  for (int k0 = 0; k0 < K; k0 += BK) {
+  for (int k0 = k_lo; k0 < K; k0 += BK) {
     const bool more = k0 + BK < K;
     if (more) fetch(k0 + BK);
 #pragma unroll
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
   __shared__ __attribute__((aligned(16))) bf16 xs[MB > 1 ? MB * 16 * XS_STRIDE : 8];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int nb = (blockIdx.x * 4 + wave) * 16;
+  const int nb = (blockIdx.x * (blockDim.x / WAVE) + wave) * 16;  // MB == 1 runs one wave per block
   const int n = nb + r;
   const int k_begin = blockIdx.y * steps_per_split * 64;
   const int k_end = min(K, k_begin + steps_per_split * 64);
@@ -282,7 +287,9 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   dim3 grid((N + 63) / 64, splits);
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
-  if (M <= 16) gemm_bf16_small_kernel<1><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
+  // Without a shared X slab the waves of a block have nothing in common: single-wave blocks spread
+  // evenly over the CUs.
+  if (M <= 16) gemm_bf16_small_kernel<1><<<dim3((N + 15) / 16, splits), WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per);
   else if (M <= 32) gemm_bf16_small_kernel<2><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
   else gemm_bf16_small_kernel<4><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
   if (reduce) {
@@ -292,23 +299,40 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   return launch_status();
 }
 
+// Splits of K for the tile kernel when the caller takes partial sums: as many as fill the chip with
+// 128 x 128 tiles (at most 4), each at least 512 k long.
+extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
+  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles >= 256) return 1;
+  int s = (int)((256 + tiles - 1) / tiles);
+  if (s > 4) s = 4;
+  while (s > 1 && K / s < 512) --s;
+  return s;
+}
+
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
+// splits > 1 (mode 1 only): C holds splits * M * N floats of partial sums, slice after slice.
 extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,
-                            hipStream_t st) {
+                            int splits, hipStream_t st) {
   if (M <= 0 || N <= 0) return MS_OK;
-  if (K <= 0 || ldx < K || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
+  if (K <= 0 || ldx < K || ldc < N || mode < 0 || mode > 2 || splits < 1 || (splits > 1 && (mode != 1 || ldc != N)))
+    return MS_BAD_ARG;
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
+  const int k_per = ((K + splits - 1) / splits + BK - 1) / BK * BK;
+  const int nz = (K + k_per - 1) / k_per;
+  if (nz != splits) return MS_BAD_ARG;  // the caller sized C for `splits` slices
+  const size_t stride = (size_t)M * N;
   // Large tiles when they still give every CU work; small tiles otherwise.
-  const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const long big = (long)((M + 127) / 128) * ((N + 127) / 128) * splits;
   if (big >= 256) {
-    dim3 grid((N + 127) / 128, (M + 127) / 128);
+    dim3 grid((N + 127) / 128, (M + 127) / 128, splits);
     if (grid.y > 65535) return MS_BAD_ARG;
-    gemm_bf16_tile_kernel<128, 128><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+    gemm_bf16_tile_kernel<128, 128><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
   } else {
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    dim3 grid((N + 63) / 64, (M + 63) / 64, splits);
     if (grid.y > 65535) return MS_BAD_ARG;
-    gemm_bf16_tile_kernel<64, 64><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc);
+    gemm_bf16_tile_kernel<64, 64><<<grid, 256, 0, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
   }
   return launch_status();
 }

@@ -30,7 +30,8 @@ _SIGNATURES = {
                               _c_int, _c_float, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16_tile_splits": [_c_int, _c_int, _c_int],
     "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_small_splits": [_c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -38,9 +39,9 @@ _SIGNATURES = {
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
-    "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void,
-                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
-    "ms_attention_prefill_tile_tokens": [_c_int],
+    "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
+                                  _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
 }
 
@@ -253,6 +254,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
         _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), out.data_ptr(), mode, 1, m, n, k,
                                       k, n, _stream()), "gemm_bf16_small")
         return None if accumulate_into is not None else out
+    if weight.dtype == BF16 and defer:
+        splits = lib.ms_gemm_bf16_tile_splits(m, n, k)
+        if splits > 1:  # few output tiles: split K over the grid and leave the sum to the consumer
+            xa = cast(x, BF16)
+            parts = torch.empty((splits, m, n), dtype=F32, device=x.device)
+            _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), 1, m, n, k, k, n, splits, _stream()),
+                   "gemm_bf16")
+            return SplitSum(parts)
     out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
     if weight.dtype == F32:
         xa = cast(x, F32)
@@ -261,7 +270,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
     else:
         xa = cast(x, BF16)
         mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
-        _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()), "gemm_bf16")
+        _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, 1, _stream()), "gemm_bf16")
     return None if accumulate_into is not None else out
 
 
@@ -349,6 +358,7 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
     return page
 
 
+PREFILL_ROWS = 64  # query rows (tokens x group heads) per block of the prefill attention kernel
 DECODE_TARGET_BLOCKS = 1024  # workgroups the split decode kernel aims for
 DECODE_MIN_CHUNKS = 2  # 32-token chunks a split should at least hold
 
@@ -405,10 +415,13 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             _ptr(part_o), _ptr(part_ml), n_dec, splits, num_heads, num_kv_heads, head_dim, page, float(scale), int(window),
             _stream()), "attention_decode")
     if n_dec < t:
-        first, count, tiles = batch.prefill_tiles(lib.ms_attention_prefill_tile_tokens(num_heads // num_kv_heads))
+        group = num_heads // num_kv_heads
+        rows = PREFILL_ROWS if group <= PREFILL_ROWS else 128
+        first, count, tiles = batch.prefill_tiles(lib.ms_attention_prefill_tile_tokens(group, rows))
         _check(lib.ms_attention_prefill_bf16(
             qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(),
-            tiles, *meta, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_prefill")
+            tiles, rows, *meta, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()),
+            "attention_prefill")
     return out
 
 

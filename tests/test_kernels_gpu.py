@@ -155,6 +155,21 @@ def test_pending_sums_feed_their_consumers(ops, m):
     close(r4, full, 1e-5, "accumulate")
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 4), (2048, 1024, 3072, 2), (300, 1000, 1100, 2), (2048, 4096, 1024, 1)])
+def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
+    x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
+    want = x.double() @ w.double().T
+    resid = rand((m, n), F32, 62)
+    r = resid.clone()
+    pend = ops.linear(x, w, accumulate_into=r, defer=True)
+    if splits == 1:
+        assert pend is None
+    else:
+        assert isinstance(pend, ops.SplitSum) and pend.splits == splits and torch.equal(r, resid)
+        ops.add_pending(r, pend)
+    close(r, resid.double() + want, 1e-5, "tile product with split K")
+
+
 def test_linear_with_float32_weights_in_bfloat16_mode(ops):
     x, w = rand((9, 96), BF16, 14), rand((50, 96), F32, 15)
     close(ops.linear(x, w, out_dtype=BF16), x.double() @ w.double().T, 5e-3, "f32 weights, bf16 activations")
