@@ -84,7 +84,9 @@ extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y
                           int width, float eps, const float* parts, int splits, long long split_stride, hipStream_t st) {
   if (n_rows <= 0) return MS_OK;
   if (width <= 0 || (parts != nullptr && splits < 1)) return MS_BAD_ARG;
-  const bool wide = n_rows <= 256;
+  // float32 output keeps one block shape for every batch, so that its sums are formed in one order
+  // whatever the batch; bfloat16 output takes the wide block for few rows.
+  const bool wide = y_is_bf16 && n_rows <= 256;
 #define LAUNCH(TW, TO)                                                                                                  \
   if (wide)                                                                                                             \
     rmsnorm_kernel<TW, TO, 1024, 4><<<n_rows, 1024, 0, st>>>(x, (const TW*)w, (TO*)y, rows, width, eps, parts, splits,  \

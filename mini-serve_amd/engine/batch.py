@@ -83,7 +83,8 @@ class BatchBuilder:
         lens = [len(r.tokens) for r in rows]
         T = sum(lens)
         n_want = sum(len(r.want) for r in rows)
-        widths = [max(1, max(r.cache.tables[g].num_blocks for r in rows)) for g in range(self.num_groups)]
+        # table rows are a multiple of 4 entries wide: kernels fetch the page ids of a key tile with one 16-byte load
+        widths = [_align(max(1, max(r.cache.tables[g].num_blocks for r in rows))) for g in range(self.num_groups)]
 
         seg = {}
         off = 0

@@ -358,7 +358,7 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
     return page
 
 
-PREFILL_ROWS = 64  # query rows (tokens x group heads) per block of the prefill attention kernel
+PREFILL_BIG_BLOCKS = 1024  # from this many 128-row blocks on, the prefill attention runs 128-row blocks
 DECODE_TARGET_BLOCKS = 1024  # workgroups the split decode kernel aims for
 DECODE_MIN_CHUNKS = 2  # 32-token chunks a split should at least hold
 
@@ -415,8 +415,16 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             _ptr(part_o), _ptr(part_ml), n_dec, splits, num_heads, num_kv_heads, head_dim, page, float(scale), int(window),
             _stream()), "attention_decode")
     if n_dec < t:
+        if block_table.shape[1] % 4:  # the prefill kernel reads four page ids at once
+            wide = torch.zeros((block_table.shape[0], -(-block_table.shape[1] // 4) * 4), dtype=I32, device=block_table.device)
+            wide[:, : block_table.shape[1]] = block_table
+            block_table = wide
+            common = (block_table.data_ptr(), block_table.shape[1])
         group = num_heads // num_kv_heads
-        rows = PREFILL_ROWS if group <= PREFILL_ROWS else 128
+        # 128 query rows per block read K and V least often; 64 (each wave takes half of every key tile)
+        # give short chains and more blocks. The latter until 128-row blocks alone fill the chip twice over.
+        n_prefill = t - n_dec
+        rows = 128 if (group > 64 or -(-n_prefill // (128 // group)) * num_kv_heads >= PREFILL_BIG_BLOCKS) else 64
         first, count, tiles = batch.prefill_tiles(lib.ms_attention_prefill_tile_tokens(group, rows))
         _check(lib.ms_attention_prefill_bf16(
             qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(),
