@@ -115,7 +115,7 @@ def main() -> int:
     del eng
 
     out = {
-        "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape, context 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-{args.preset} shape, context {args.context})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, random token ids)",

@@ -23,8 +23,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 #define PAGE 16
 #define CHUNK 32  // tokens per step of a wave: two pages
 
+// Keys and values of one 32-token chunk as a wave holds them: the matrix operands themselves.
 template <int D>
-__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+struct DecodeTile {
+  bf16x8 ka[D / 32], kb[D / 32];
+  bf16x4 va[D / 16], vb[D / 16];
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tokens,
     const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
@@ -63,45 +70,44 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
 #pragma unroll
   for (int i = 0; i < DB; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // Page ids of a chunk are fetched one iteration ahead, so that their latency is not in the chain
-  // table -> page -> keys of every iteration.
+  // Two chunks are in flight per wave: while one is multiplied the next one's keys and values are
+  // already on their way, and the page ids of the one after that. Loads go out in chunk order, so
+  // one pair of prefetched page ids is enough.
   int p0n = 0, p1n = 0;
-  if (c_begin + wave < c_end) {
-    const int t0 = lo_al + (c_begin + wave) * CHUNK;
-    p0n = table[t0 / PAGE];
-    p1n = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0n;
-  }
-  for (int c = c_begin + wave; c < c_end; c += 4) {
-    const int t0 = lo_al + c * CHUNK;
+  auto fetch_ids = [&](int c) {
+    if (c < c_end) {
+      const int t0 = lo_al + c * CHUNK;
+      p0n = table[t0 / PAGE];
+      p1n = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0n;
+    }
+  };
+  auto load = [&](DecodeTile<D>& t, int c) {
     const int p0 = max(p0n, 0);  // a page behind the window was given back: its tokens are masked below
     const int p1 = max(p1n, 0);
-    if (c + 4 < c_end) {
-      const int tn = t0 + 4 * CHUNK;
-      p0n = table[tn / PAGE];
-      p1n = (tn + PAGE < kv_len) ? table[tn / PAGE + 1] : p0n;
-    }
+    fetch_ids(c + 4);
     const bf16* k0 = kc + (((size_t)p0 * Hkv + kvh) * PAGE + r) * D + g * 8;
     const bf16* k1 = kc + (((size_t)p1 * Hkv + kvh) * PAGE + r) * D + g * 8;
-    bf16x8 ka[KK], kb[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      ka[kk] = *reinterpret_cast<const bf16x8*>(k0 + kk * 32);
-      kb[kk] = *reinterpret_cast<const bf16x8*>(k1 + kk * 32);
+      t.ka[kk] = *reinterpret_cast<const bf16x8*>(k0 + kk * 32);
+      t.kb[kk] = *reinterpret_cast<const bf16x8*>(k1 + kk * 32);
     }
     // V^T operand: element d = db * 16 + r, tokens 4 g .. 4 g + 3 of each page.
     const bf16* v0 = vc + (((size_t)p0 * Hkv + kvh) * D + r) * PAGE + g * 4;
     const bf16* v1 = vc + (((size_t)p1 * Hkv + kvh) * D + r) * PAGE + g * 4;
-    bf16x4 va[DB], vb[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      va[db] = *reinterpret_cast<const bf16x4*>(v0 + (size_t)db * 16 * PAGE);
-      vb[db] = *reinterpret_cast<const bf16x4*>(v1 + (size_t)db * 16 * PAGE);
+      t.va[db] = *reinterpret_cast<const bf16x4*>(v0 + (size_t)db * 16 * PAGE);
+      t.vb[db] = *reinterpret_cast<const bf16x4*>(v1 + (size_t)db * 16 * PAGE);
     }
+  };
+  auto multiply = [&](const DecodeTile<D>& t, int c) {
+    const int t0 = lo_al + c * CHUNK;
     floatx4 s0 = floatx4{0.f, 0.f, 0.f, 0.f}, s1 = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], qf[kk], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[kk], qf[kk], s1, 0, 0, 0);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.ka[kk], qf[kk], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.kb[kk], qf[kk], s1, 0, 0, 0);
     }
     // This lane: tokens t0 + 4 g + i (s0) and t0 + 16 + 4 g + i (s1) of query r.
     float sc[8];
@@ -141,10 +147,25 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
       bf16x8 vf;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        vf[i] = va[db][i];
-        vf[4 + i] = vb[db][i];
+        vf[i] = t.va[db][i];
+        vf[4 + i] = t.vb[db][i];
       }
       o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+    }
+  };
+  {
+    DecodeTile<D> ta, tb;
+    int c = c_begin + wave;
+    fetch_ids(c);
+    if (c < c_end) load(ta, c);
+    while (c < c_end) {
+      if (c + 4 < c_end) load(tb, c + 4);
+      multiply(ta, c);
+      c += 4;
+      if (c >= c_end) break;
+      if (c + 4 < c_end) load(ta, c + 4);
+      multiply(tb, c);
+      c += 4;
     }
   }
 

@@ -165,26 +165,31 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(const bf16* __re
 // rows and a slice of K; per step of 64 k each lane loads 32 bytes of its weight row and issues two
 // MFMAs per 16-row block of X. With MB == 1 the matching 32 bytes of an X row come straight from
 // global memory (X is a few KB and stays in the vector cache; no LDS, no barrier); with MB > 1 the
-// block's four waves stage the X slab of their common K slice in LDS. K is split over blockIdx.y so
+// block's four waves stage the X slab of their common K slice in LDS. K is split over the grid so
 // that even a 1024-row matrix gives every CU several waves; each split writes float partial sums
 // P[split, M, N], which the caller's next kernel (or the reduction below) sums in ascending split
-// order. The number of splits depends on N and K alone, never on M: a row's result does not depend on
-// the batch it is in (within the same MB).
+// order. The number of splits depends on N, K and on whether M is above 16, not on M itself: a row's
+// result does not depend on the batch it is in (within the same MB).
 #define SMALL_SLAB 256  // k per iteration: four steps of 64
 #define XS_STRIDE (SMALL_SLAB + 8)
 
 template <int MB>
 __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                               float* __restrict__ P, int M, int N, int K, int ldx,
-                                                              int steps_per_split) {
+                                                              int steps_per_split, int splits) {
   __shared__ __attribute__((aligned(16))) bf16 xs[MB > 1 ? MB * 16 * XS_STRIDE : 8];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int nb = (blockIdx.x * (blockDim.x / WAVE) + wave) * 16;  // MB == 1 runs one wave per block
+  // The split index runs fastest over the grid: blocks that are resident together read neighbouring
+  // k ranges of the same weight rows, which together are whole rows, instead of the same k range of
+  // rows that lie a power of two apart (those would queue up on a few memory channels).
+  const int split = blockIdx.x % splits, row_block = blockIdx.x / splits;
+  const int nb = (row_block * (blockDim.x / WAVE) + wave) * 16;  // MB == 1 runs one wave per block
   const int n = nb + r;
-  const int k_begin = blockIdx.y * steps_per_split * 64;
+  const int k_begin = split * steps_per_split * 64;
   const int k_end = min(K, k_begin + steps_per_split * 64);
   const bool vecx = (K % 8 == 0) && (ldx % 8 == 0), vecw = (K % 8 == 0);
+  const bool rows_in = vecw && nb + 16 <= N;  // the same for the whole wave
 
   floatx4 acc[MB];
 #pragma unroll
@@ -192,23 +197,46 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
 
   for (int k0 = k_begin; k0 < k_end; k0 += SMALL_SLAB) {
     // This lane's weights of the slab: per step of 64 k, 16 consecutive k at offset 16 g. Chunks at or
-    // beyond k_end are asked for at K, where load_chunk yields zeros.
+    // beyond k_end are asked for at K, where load_chunk yields zeros. A slab that lies wholly inside
+    // the matrix is loaded without any test, so that all its loads go out back to back.
+    const bool whole = k0 + SMALL_SLAB <= k_end;
     Chunk w[SMALL_SLAB / 64][2];
+    if (rows_in && whole) {
+      const bf16* wp = W + (size_t)n * K + k0 + g * 16;
 #pragma unroll
-    for (int u = 0; u < SMALL_SLAB / 64; ++u) {
-      const int k = k0 + u * 64 + g * 16;
-      const int kw = k < k_end ? k : K;
-      w[u][0] = load_chunk(W, n, N, kw, K, K, vecw);
-      w[u][1] = load_chunk(W, n, N, kw + 8, K, K, vecw);
-    }
-    if (MB == 1) {
-      Chunk x[SMALL_SLAB / 64][2];
+      for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+        w[u][0].u = *reinterpret_cast<const uint4*>(wp + u * 64);
+        w[u][1].u = *reinterpret_cast<const uint4*>(wp + u * 64 + 8);
+      }
+    } else {
 #pragma unroll
       for (int u = 0; u < SMALL_SLAB / 64; ++u) {
         const int k = k0 + u * 64 + g * 16;
         const int kw = k < k_end ? k : K;
-        x[u][0] = load_chunk(X, r, M, kw, K, ldx, vecx);
-        x[u][1] = load_chunk(X, r, M, kw + 8, K, ldx, vecx);
+        w[u][0] = load_chunk(W, n, N, kw, K, K, vecw);
+        w[u][1] = load_chunk(W, n, N, kw + 8, K, K, vecw);
+      }
+    }
+    if (MB == 1) {
+      Chunk x[SMALL_SLAB / 64][2];
+      if (vecx && whole) {
+        const bf16* xp = X + (size_t)min(r, M - 1) * ldx + k0 + g * 16;  // rows beyond M: read row M - 1, use zeros
+        const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+          const uint4 a = *reinterpret_cast<const uint4*>(xp + u * 64);
+          const uint4 b = *reinterpret_cast<const uint4*>(xp + u * 64 + 8);
+          x[u][0].u = r < M ? a : zero;
+          x[u][1].u = r < M ? b : zero;
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+          const int k = k0 + u * 64 + g * 16;
+          const int kw = k < k_end ? k : K;
+          x[u][0] = load_chunk(X, r, M, kw, K, ldx, vecx);
+          x[u][1] = load_chunk(X, r, M, kw + 8, K, ldx, vecx);
+        }
       }
 #pragma unroll
       for (int u = 0; u < SMALL_SLAB / 64; ++u) {
@@ -238,7 +266,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
     }
   }
   // acc[i][e] = C[m = 16 i + r][n = nb + 4 g + e]
-  float* dst = P + (size_t)blockIdx.y * M * N;
+  float* dst = P + (size_t)split * M * N;
 #pragma unroll
   for (int i = 0; i < MB; ++i) store4(dst, 1, i * 16 + r, nb + g * 4, M, N, N, acc[i], N % 4 == 0);
 }
@@ -263,15 +291,23 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
 }
 
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
-// its loads at once, unless that would make more than about 8192 waves (then longer slices).
-extern "C" int ms_gemm_bf16_small_splits(int N, int K) {
-  const int steps = (K + 63) / 64;
+// its loads at once, unless that would make more waves than the chip holds a few times over (then
+// slices of several whole slabs). With up to 16 rows the partial sums are small beside the weights
+// and 32768 waves are allowed; above that 8192. The count depends on M only through that class.
+static int small_slabs_per_split(int M, int N, int K) {
+  const int slabs = (K + SMALL_SLAB - 1) / SMALL_SLAB;
   const int row_blocks = (N + 15) / 16;
-  int s = (steps + 3) / 4;
-  const int most = 8192 / row_blocks > 0 ? 8192 / row_blocks : 1;
+  const int waves = M <= 16 ? 32768 : 8192;
+  int s = slabs;
+  const int most = waves / row_blocks > 0 ? waves / row_blocks : 1;
   if (s > most) s = most;
-  const int per = (steps + s - 1) / s;
-  return (steps + per - 1) / per;  // no empty split
+  return (slabs + s - 1) / s;
+}
+
+extern "C" int ms_gemm_bf16_small_splits(int M, int N, int K) {
+  const int slabs = (K + SMALL_SLAB - 1) / SMALL_SLAB;
+  const int per = small_slabs_per_split(M, N, K);
+  return (slabs + per - 1) / per;  // no empty split
 }
 
 // X [M <= 64, K] * W [N, K]^T. `partials` holds splits * M * N floats (splits from
@@ -281,17 +317,17 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
                                   int N, int K, int ldx, int ldc, hipStream_t st) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64 || K <= 0 || ldx < K || partials == nullptr) return MS_BAD_ARG;
-  const int splits = ms_gemm_bf16_small_splits(N, K);
-  const int steps = (K + 63) / 64;
-  const int per = (steps + splits - 1) / splits;
-  dim3 grid((N + 63) / 64, splits);
+  const int splits = ms_gemm_bf16_small_splits(M, N, K);
+  const int per = small_slabs_per_split(M, N, K) * (SMALL_SLAB / 64);
+  const long wave_blocks = (long)((N + 15) / 16) * splits, wide_blocks = (long)((N + 63) / 64) * splits;
+  if (wave_blocks > 0x7fffffffL) return MS_BAD_ARG;
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
   // Without a shared X slab the waves of a block have nothing in common: single-wave blocks spread
   // evenly over the CUs.
-  if (M <= 16) gemm_bf16_small_kernel<1><<<dim3((N + 15) / 16, splits), WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per);
-  else if (M <= 32) gemm_bf16_small_kernel<2><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
-  else gemm_bf16_small_kernel<4><<<grid, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per);
+  if (M <= 16) gemm_bf16_small_kernel<1><<<(unsigned)wave_blocks, WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  else if (M <= 32) gemm_bf16_small_kernel<2><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  else gemm_bf16_small_kernel<4><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
   if (reduce) {
     if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
     splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);

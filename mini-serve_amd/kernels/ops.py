@@ -33,7 +33,7 @@ _SIGNATURES = {
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_tile_splits": [_c_int, _c_int, _c_int],
     "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_gemm_bf16_small_splits": [_c_int, _c_int],
+    "ms_gemm_bf16_small_splits": [_c_int, _c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
@@ -238,7 +238,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
     lib = library()
     if weight.dtype == BF16 and m <= SMALL_M:
         xa = cast(x, BF16)
-        splits = lib.ms_gemm_bf16_small_splits(n, k)
+        splits = lib.ms_gemm_bf16_small_splits(m, n, k)
         if splits == 1 and accumulate_into is None and out_dtype == F32:
             out = torch.empty((m, n), dtype=F32, device=x.device)  # the single partial sum is the result
             _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), None, 1, 0, m, n, k, k, n,
@@ -359,8 +359,8 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
 
 
 PREFILL_BIG_BLOCKS = 1024  # from this many 128-row blocks on, the prefill attention runs 128-row blocks
-DECODE_TARGET_BLOCKS = 1024  # workgroups the split decode kernel aims for
-DECODE_MIN_CHUNKS = 2  # 32-token chunks a split should at least hold
+DECODE_TARGET_BLOCKS = 512  # workgroups the split decode kernel aims for
+DECODE_MIN_CHUNKS = 4  # 32-token chunks a split should at least hold
 
 
 def decode_splits(rows: int, num_kv_heads: int, max_kv_len: int) -> int:

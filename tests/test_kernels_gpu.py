@@ -368,8 +368,8 @@ def test_prefill_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost
 
 
 def test_decode_splits_rule(ops):
-    assert ops.decode_splits(1, 8, 4096) == 64 and ops.decode_splits(8, 8, 4096) == 16 and ops.decode_splits(64, 8, 4096) == 2
-    assert ops.decode_splits(1, 8, 100) == 2 and ops.decode_splits(1, 1, 40000) == 625 and ops.decode_splits(1, 8, 1) == 1
+    assert ops.decode_splits(1, 8, 4096) == 32 and ops.decode_splits(8, 8, 4096) == 8 and ops.decode_splits(64, 8, 4096) == 1
+    assert ops.decode_splits(1, 8, 100) == 1 and ops.decode_splits(1, 1, 40000) == 312 and ops.decode_splits(1, 8, 1) == 1
 
 
 def test_attention_one_token_returns_its_value(ops):
