@@ -163,35 +163,50 @@ extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf1
 }
 
 // ---------------------------------------------------------------------------------------------
-// One block of 4 waves per (token, four head slots): a wave per head slot. Head slots [0, Hq)
-// are query heads, [Hq, Hq+Hkv) key heads, [Hq+Hkv, Hq+2Hkv) value heads of the token's row in
-// qkv [tokens, (Hq + 2 Hkv) * D].
+// Cosines and sines of a step's rotation angles, table [tokens, 2 * half]: cos(a) in the first half of
+// a row, sin(a) in the second, a = float(pos[t]) * inv_freq[j]. Made once per step and read by every
+// layer's rotation kernel.
+__global__ void rope_table_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq, float* __restrict__ out,
+                                  int tokens, int half) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= tokens * half) return;
+  const int t = i / half, j = i % half;
+  float sn, cs;
+  sincosf((float)pos[t] * inv_freq[j], &sn, &cs);
+  out[(size_t)t * 2 * half + j] = cs;
+  out[(size_t)t * 2 * half + half + j] = sn;
+}
+
+extern "C" int ms_rope_table(const int* pos, const float* inv_freq, float* out, int tokens, int half, hipStream_t st) {
+  if (tokens <= 0 || half <= 0) return MS_OK;
+  if ((long long)tokens * half > 0x7fffffffLL) return MS_BAD_ARG;
+  rope_table_kernel<<<(tokens * half + 255) / 256, 256, 0, st>>>(pos, inv_freq, out, tokens, half);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Head slots [0, Hq) are query heads, [Hq, Hq+Hkv) key heads, [Hq+Hkv, Hq+2Hkv) value heads of the
+// token's row in qkv [tokens, (Hq + 2 Hkv) * D].
 //   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
-//         pairs (j, j + rot/2) by angle float(pos) * inv_freq[j] (sine and cosine are formed once per
-//         block and shared by its four heads);
+//         pairs (j, j + rot/2) by the angle whose cosine and sine are rope[t][j] and rope[t][rot/2 + j];
 //   q goes to q_out; k and v go to the cache page of the token's slot
 //   (slot = page * page_size + offset; keys [pages, Hkv, page_size, D], values transposed within
 //   the page, [pages, Hkv, D, page_size]).
 // With slots == nullptr only the query heads are processed (the entry reads another entry's cache).
+//
+// General kernel (any head size up to 256, rotation over part of the head): one block of 4 waves per
+// (token, four head slots), a wave per head slot.
 #define MAX_HEAD_DIM 256
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const T* qkv, const float* __restrict__ parts, int splits, size_t split_stride, T* q_out, int q_out_stride,
-    const int* __restrict__ pos, const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw,
-    float eps, const float* __restrict__ inv_freq, int rot, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D,
-    int page_size, int heads) {
-  __shared__ float cs[MAX_HEAD_DIM / 2], sn[MAX_HEAD_DIM / 2];
+    const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
+    const float* __restrict__ rope, int rot, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D, int page_size,
+    int heads) {
   __shared__ float buf[4][MAX_HEAD_DIM];
   const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int hs = blockIdx.y * 4 + wave;  // this wave's head slot
   const int half = rot / 2;
-  if (threadIdx.x < half) {
-    float s, c;
-    sincosf((float)pos[t] * inv_freq[threadIdx.x], &s, &c);
-    cs[threadIdx.x] = c;
-    sn[threadIdx.x] = s;
-  }
-  __syncthreads();
   constexpr int PER = MAX_HEAD_DIM / WAVE;
   if (hs < heads) {
     const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);
@@ -236,6 +251,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
       if (rot > 0) {
         // The wave exchanges the partners of its pairs through its own LDS row; a wave runs in
         // lockstep, so no block barrier is needed between its write and its read.
+        const float* cs = rope + (size_t)t * rot;
+        const float* sn = cs + half;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
           const int e = lane + i * WAVE;
@@ -261,24 +278,185 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   }
 }
 
+// D = 64 or 128, rotation over the whole head or none: one block per
+// (256 / (D/8) consecutive tokens, head slot). A thread owns 8 consecutive elements of one token's
+// head, moved as one vector; the D/8 threads of a token are neighbours in a wave and share the sum of
+// squares and the rotation partners (thread i and thread i ^ D/16) through lane exchanges. Value
+// heads are turned in LDS so that a thread writes 8 consecutive tokens of one head element with one
+// vector store where those tokens fill an aligned run of a page (single stores otherwise).
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<bf16> {
+  uint4 raw;
+  __device__ __forceinline__ void load(const bf16* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void store(bf16* p) const { *reinterpret_cast<uint4*>(p) = raw; }
+  __device__ __forceinline__ float get(int i) const { return to_f32(reinterpret_cast<const bf16*>(&raw)[i]); }
+  __device__ __forceinline__ void set(int i, float v) { reinterpret_cast<bf16*>(&raw)[i] = from_f32<bf16>(v); }
+};
+template <>
+struct Vec8<float> {
+  float4 lo, hi;
+  __device__ __forceinline__ void load(const float* p) {
+    lo = *reinterpret_cast<const float4*>(p);
+    hi = *reinterpret_cast<const float4*>(p + 4);
+  }
+  __device__ __forceinline__ void store(float* p) const {
+    *reinterpret_cast<float4*>(p) = lo;
+    *reinterpret_cast<float4*>(p + 4) = hi;
+  }
+  __device__ __forceinline__ float get(int i) const { return i < 4 ? (&lo.x)[i] : (&hi.x)[i - 4]; }
+  __device__ __forceinline__ void set(int i, float v) {
+    if (i < 4) (&lo.x)[i] = v;
+    else (&hi.x)[i - 4] = v;
+  }
+};
+
+template <typename T, typename TW, int D>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_tile_kernel(
+    const T* qkv, const float* __restrict__ parts, int splits, size_t split_stride, T* q_out, int q_out_stride,
+    const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
+    const float* __restrict__ rope, T* __restrict__ kc, T* __restrict__ vc, int tokens, int Hq, int Hkv, int page_size) {
+  constexpr int TPT = D / 8;      // threads per token
+  constexpr int TOK = 256 / TPT;  // tokens per block
+  constexpr int RUNS = TOK / 8;   // runs of 8 tokens
+  __shared__ __attribute__((aligned(16))) T vt[TOK][D + 8];
+  const int hs = blockIdx.y;
+  const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);  // the same for the whole block
+  const int tl = threadIdx.x / TPT, i = threadIdx.x % TPT;
+  const int t0 = blockIdx.x * TOK, t = t0 + tl;
+  const bool live = t < tokens;
+  const size_t at = ((size_t)(live ? t : tokens - 1) * (Hq + 2 * Hkv) + hs) * D + i * 8;
+
+  float x[8];
+  if (parts != nullptr) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = 0.f;
+    for (int s = 0; s < splits; ++s) {  // ascending split order; the two loads of a split go out together
+      const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)s * split_stride + at);
+      const float4 b = *reinterpret_cast<const float4*>(parts + (size_t)s * split_stride + at + 4);
+      x[0] += a.x; x[1] += a.y; x[2] += a.z; x[3] += a.w;
+      x[4] += b.x; x[5] += b.y; x[6] += b.z; x[7] += b.w;
+    }
+  } else {
+    Vec8<T> v;
+    v.load(qkv + at);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = v.get(e);
+  }
+
+  if (kind != 2) {
+    const TW* w = kind == 0 ? qw : kw;
+    if (w != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+      for (int o = 1; o < TPT; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+      const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = x[e] * rstd * to_f32(w[i * 8 + e]);
+    }
+    if (rope != nullptr) {
+      const int j0 = (i % (TPT / 2)) * 8;
+      const float* cs = rope + (size_t)(live ? t : tokens - 1) * D + j0;
+      const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2), s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
+      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+      const bool low = i < TPT / 2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float partner = __shfl_xor(x[e], TPT / 2, WAVE);
+        x[e] = low ? x[e] * c[e] - partner * sn[e] : x[e] * c[e] + partner * sn[e];
+      }
+    }
+    if (live) {
+      Vec8<T> v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v.set(e, x[e]);
+      if (kind == 0) {
+        v.store(q_out + (size_t)t * q_out_stride + (size_t)hs * D + i * 8);
+      } else {
+        const int s = slots[t];
+        v.store(kc + (((size_t)(s / page_size) * Hkv + (hs - Hq)) * page_size + (s % page_size)) * D + i * 8);
+      }
+    }
+    return;
+  }
+
+  // Value head: through LDS, then thread (d, run) writes tokens 8 run .. 8 run + 7 of head element d.
+  {
+    Vec8<T> v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v.set(e, x[e]);
+    v.store(&vt[tl][i * 8]);
+  }
+  __syncthreads();
+  const int d = threadIdx.x / RUNS, run = threadIdx.x % RUNS;
+  const int tr = t0 + run * 8;
+  if (tr >= tokens) return;
+  const int kvh = hs - Hq - Hkv;
+  const int n_live = min(8, tokens - tr);
+  int sl[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sl[e] = slots[min(tr + e, tokens - 1)];
+  bool run_ok = n_live == 8 && (page_size % 8 == 0) && (sl[0] % 8 == 0);
+#pragma unroll
+  for (int e = 1; e < 8; ++e) run_ok = run_ok && sl[e] == sl[0] + e;
+  if (run_ok) {
+    Vec8<T> v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v.set(e, to_f32(vt[run * 8 + e][d]));
+    v.store(vc + (((size_t)(sl[0] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[0] % page_size));
+  } else {
+    for (int e = 0; e < n_live; ++e)
+      vc[(((size_t)(sl[e] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[e] % page_size)] = vt[run * 8 + e][d];
+  }
+}
+
 // Source: qkv [tokens, (Hq + 2 Hkv) D], or (parts != nullptr) float partial sums [splits, tokens, (Hq + 2 Hkv) D] of it.
-// Queries go to q_out [tokens, q_out_stride >= Hq D] (which may be qkv itself: in place).
+// Queries go to q_out [tokens, q_out_stride >= Hq D] (which may be qkv itself: in place). rope is the
+// table of ms_rope_table for these tokens with half = rot / 2 (nullptr when rot == 0).
 extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int splits, long long split_stride, void* q_out,
-                                     int q_out_stride, int is_bf16, const int* pos, const int* slots, const void* qw,
-                                     const void* kw, int w_is_bf16, float eps, const float* inv_freq, int rot, void* kc,
-                                     void* vc, int tokens, int Hq, int Hkv, int D, int page_size, hipStream_t st) {
+                                     int q_out_stride, int is_bf16, const int* slots, const void* qw, const void* kw,
+                                     int w_is_bf16, float eps, const float* rope, int rot, void* kc, void* vc, int tokens,
+                                     int Hq, int Hkv, int D, int page_size, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if ((qkv == nullptr) == (parts == nullptr) || (parts != nullptr && splits < 1) || q_out == nullptr || q_out_stride < Hq * D)
     return MS_BAD_ARG;
   if (D <= 0 || D > MAX_HEAD_DIM || rot < 0 || rot > D || (rot & 1) || Hq <= 0 || Hkv <= 0 || page_size <= 0) return MS_BAD_ARG;
   if ((qw == nullptr) != (kw == nullptr)) return MS_BAD_ARG;
-  if (rot > 0 && inv_freq == nullptr) return MS_BAD_ARG;
+  if ((rot > 0) != (rope != nullptr)) return MS_BAD_ARG;
   const int heads = slots ? Hq + 2 * Hkv : Hq;
-  if ((heads + 3) / 4 > 65535) return MS_BAD_ARG;
+  if ((heads + 3) / 4 > 65535 || heads > 65535) return MS_BAD_ARG;
+  // The tile kernel moves 8 elements at a time: every row it touches must start on such a boundary.
+  // Which kernel runs depends on the head's shape alone, never on the number of tokens: a token's
+  // result is the same bit for bit in whatever step it comes.
+  const bool tiled = (D == 64 || D == 128) && (rot == 0 || rot == D) && q_out_stride % 8 == 0 &&
+                     (parts == nullptr || split_stride % 4 == 0);
+  if (tiled) {
+    const int tok_per_block = 256 / (D / 8);
+    const dim3 grid((tokens + tok_per_block - 1) / tok_per_block, heads);
+#define LAUNCH_TILE(T, TW, DD)                                                                                          \
+  qk_norm_rope_store_tile_kernel<T, TW, DD><<<grid, 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride,   \
+                                                                   (T*)q_out, q_out_stride, slots, (const TW*)qw,        \
+                                                                   (const TW*)kw, eps, rope, (T*)kc, (T*)vc, tokens, Hq, \
+                                                                   Hkv, page_size)
+#define LAUNCH_TILE_D(T, TW) \
+  if (D == 128) LAUNCH_TILE(T, TW, 128); else LAUNCH_TILE(T, TW, 64)
+    if (is_bf16 && w_is_bf16) { LAUNCH_TILE_D(bf16, bf16); }
+    else if (is_bf16) { LAUNCH_TILE_D(bf16, float); }
+    else if (w_is_bf16) { LAUNCH_TILE_D(float, bf16); }
+    else { LAUNCH_TILE_D(float, float); }
+#undef LAUNCH_TILE_D
+#undef LAUNCH_TILE
+    return launch_status();
+  }
 #define LAUNCH(T, TW)                                                                                                   \
-  qk_norm_rope_store_kernel<T, TW><<<dim3(tokens, (heads + 3) / 4), 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, \
-                                                            q_out_stride, pos, slots, (const TW*)qw, (const TW*)kw, eps,  \
-                                                            inv_freq, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
+  qk_norm_rope_store_kernel<T, TW><<<dim3(tokens, (heads + 3) / 4), 256, 0, st>>>(                                      \
+      (const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, q_out_stride, slots, (const TW*)qw, (const TW*)kw, \
+      eps, rope, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
   if (is_bf16 && w_is_bf16) LAUNCH(bf16, bf16);
   else if (is_bf16) LAUNCH(bf16, float);
   else if (w_is_bf16) LAUNCH(float, bf16);

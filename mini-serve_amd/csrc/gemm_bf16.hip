@@ -200,6 +200,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
     // beyond k_end are asked for at K, where load_chunk yields zeros. A slab that lies wholly inside
     // the matrix is loaded without any test, so that all its loads go out back to back.
     const bool whole = k0 + SMALL_SLAB <= k_end;
+    // MB > 1: this thread's share of the X slab goes out first (it comes from the cache and is back
+    // while the weights are still on their way), so that staging it in LDS costs no waiting of its own.
+    constexpr int XPT = MB > 1 ? MB * 16 * (SMALL_SLAB / 8) / 256 : 1;  // 16-byte chunks per thread
+    Chunk xr[XPT];
+    if (MB > 1) {
+      if (vecx && whole) {
+        const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < XPT; ++j) {
+          const int c = tid + j * 256, m = c / (SMALL_SLAB / 8), kc = (c % (SMALL_SLAB / 8)) * 8;
+          const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)min(m, M - 1) * ldx + k0 + kc);
+          xr[j].u = m < M ? v : zero;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < XPT; ++j) {
+          const int c = tid + j * 256, m = c / (SMALL_SLAB / 8), kc = (c % (SMALL_SLAB / 8)) * 8;
+          const int k = k0 + kc;
+          xr[j] = load_chunk(X, m, M, k < k_end ? k : K, K, ldx, vecx);
+        }
+      }
+    }
     Chunk w[SMALL_SLAB / 64][2];
     if (rows_in && whole) {
       const bf16* wp = W + (size_t)n * K + k0 + g * 16;
@@ -245,11 +267,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
       }
     } else {
       __syncthreads();  // the previous slab has been consumed
-      for (int c = tid; c < MB * 16 * (SMALL_SLAB / 8); c += 256) {
-        const int m = c / (SMALL_SLAB / 8), kc = (c % (SMALL_SLAB / 8)) * 8;
-        const int k = k0 + kc;
-        const Chunk v = load_chunk(X, m, M, k < k_end ? k : K, K, ldx, vecx);
-        *reinterpret_cast<uint4*>(&xs[m * XS_STRIDE + kc]) = v.u;
+#pragma unroll
+      for (int j = 0; j < XPT; ++j) {
+        const int c = tid + j * 256, m = c / (SMALL_SLAB / 8), kc = (c % (SMALL_SLAB / 8)) * 8;
+        *reinterpret_cast<uint4*>(&xs[m * XS_STRIDE + kc]) = xr[j].u;
       }
       __syncthreads();
 #pragma unroll

@@ -39,8 +39,14 @@ class StepBatch:
     __slots__ = (
         "num_rows", "num_tokens", "num_wanted", "token_ids", "positions", "token_row", "row_start", "starts",
         "kv_lens", "state_slots", "want_rows", "groups", "row_lens", "row_starts_host", "max_kv_len", "is_decode",
-        "num_decode_tokens", "decode_tokens", "prefill_tokens", "_tiles",
+        "num_decode_tokens", "decode_tokens", "prefill_tokens", "_tiles", "memo",
     )
+
+    def __init__(self):
+        self._tiles = None
+        # What parts derive from the step's tokens alone and share between layers (a rotation table,
+        # say), by a key of the part's choosing. The model empties it at the start of every pass.
+        self.memo = {}
 
     def prefill_tiles(self, tile_tokens: int):
         """Tiles of at most ``tile_tokens`` consecutive new tokens of the rows that bring several

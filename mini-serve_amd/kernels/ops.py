@@ -26,7 +26,8 @@ _SIGNATURES = {
     "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
-    "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void,
+    "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+    "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
                               _c_int, _c_float, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -288,13 +289,26 @@ def add_pending(residual: torch.Tensor, pending: SplitSum | None) -> None:
 # ------------------------------------------------------------------------------------- attention
 
 
-def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq, rot_dim, k_cache, v_cache,
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """Cosines and sines of the rotation angles ``float32(position) * inv_freq[j]`` of a step's tokens:
+    float32 ``[T, 2 * len(inv_freq)]``, a row holding the cosines, then the sines. Made once per step
+    and shared by all layers that rotate by the same frequencies."""
+    _dev(positions, "positions", I32, 1)
+    _dev(inv_freq, "inv_freq", F32, 1)
+    t, half = positions.shape[0], inv_freq.shape[0]
+    out = torch.empty((t, 2 * half), dtype=F32, device=positions.device)
+    _check(library().ms_rope_table(positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), t, half, _stream()), "rope_table")
+    return out
+
+
+def qk_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cache,
                        num_heads, num_kv_heads, head_dim, out_dtype=None) -> torch.Tensor:
     """From ``qkv [T, (Hq + 2 Hkv) D]`` (a tensor, or a ``SplitSum`` of it): per-head RMSNorm of q and k
-    (if weights are given), rotation by ``positions`` (if ``inv_freq`` is given), k and v stored into
-    the cache pages at ``slots`` (skipped when ``slots`` is None). Returns the tensor that holds the
-    finished queries in its first ``Hq * D`` columns: ``qkv`` itself (written in place), or for a
-    ``SplitSum`` a new ``[T, Hq D]`` tensor of ``out_dtype``."""
+    (if weights are given), rotation of the first ``rope.shape[1]`` elements of each head by the angles
+    of ``rope`` (a ``rope_table`` of these tokens; None: no rotation), k and v stored into the cache
+    pages at ``slots`` (skipped when ``slots`` is None). Returns the tensor that holds the finished
+    queries in its first ``Hq * D`` columns: ``qkv`` itself (written in place), or for a ``SplitSum`` a
+    new ``[T, Hq D]`` tensor of ``out_dtype``."""
     width = (num_heads + 2 * num_kv_heads) * head_dim
     if isinstance(qkv, SplitSum):
         _dev(qkv.parts, "qkv", F32, 3)
@@ -312,9 +326,6 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
         dtype = qkv.dtype
         q_out = qkv
         src, parts, splits, stride = qkv.data_ptr(), None, 0, 0
-    _dev(positions, "positions", I32, 1)
-    if positions.shape[0] != t:
-        raise ValueError("one position per token is needed")
     if head_dim > 256 or head_dim < 1:
         raise ValueError(f"head_dim {head_dim} is outside the kernels' range 1..256")
     w_bf16 = 0
@@ -332,15 +343,15 @@ def qk_norm_rope_store(qkv, positions, slots, q_weight, k_weight, eps, inv_freq,
         if slots.shape[0] != t:
             raise ValueError("one slot per token is needed")
         page_size = _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim)
-    if inv_freq is not None:
-        _dev(inv_freq, "inv_freq", F32, 1)
-        if rot_dim % 2 or rot_dim > head_dim or inv_freq.shape[0] != rot_dim // 2:
-            raise ValueError(f"rotation over {rot_dim} elements needs {rot_dim // 2} frequencies and head_dim >= it")
-    else:
-        rot_dim = 0
+    rot_dim = 0
+    if rope is not None:
+        _dev(rope, "rope", F32, 2)
+        rot_dim = rope.shape[1]
+        if rope.shape[0] != t or rot_dim % 2 or rot_dim > head_dim or rot_dim < 2:
+            raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
     _check(library().ms_qk_norm_rope_store(
-        src, parts, splits, stride, q_out.data_ptr(), q_out.shape[1], int(dtype == BF16), positions.data_ptr(), _ptr(slots),
-        _ptr(q_weight), _ptr(k_weight), w_bf16, float(eps), _ptr(inv_freq), int(rot_dim),
+        src, parts, splits, stride, q_out.data_ptr(), q_out.shape[1], int(dtype == BF16), _ptr(slots),
+        _ptr(q_weight), _ptr(k_weight), w_bf16, float(eps), _ptr(rope), int(rot_dim),
         _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, t, num_heads,
         num_kv_heads, head_dim, page_size, _stream()), "qk_norm_rope_store")
     return q_out

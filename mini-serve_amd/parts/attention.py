@@ -73,11 +73,11 @@ class GQAttention(Mixer):
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
         qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
-        rot = self.position.rotation()
+        rot = self.position.rotation(batch)
         q = ops.qk_norm_rope_store(
-            qkv, batch.positions, cache.slots if cache.writes else None,
+            qkv, cache.slots if cache.writes else None,
             self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps),
-            rot.inv_freq if rot is not None else None, rot.dim if rot is not None else 0,
+            rot.table if rot is not None else None,
             cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, out_dtype=self.rt.dtype,
         )
         out = ops.paged_attention(

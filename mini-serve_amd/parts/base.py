@@ -5,7 +5,7 @@ device, kernels); it declares the tensors it needs under its own prefix and rece
 those. No part knows which model it is in. The kinds:
 
 * ``Norm``            ``forward(x_f32, rows=None, add=None) -> y``  (residual stream in, compute dtype out)
-* ``PositionEncoding`` ``rotation() -> Rotation | None``            (what a mixer's q/k are turned by)
+* ``PositionEncoding`` ``rotation(batch) -> Rotation | None``       (what a mixer's q/k are turned by in this step)
 * ``Mixer``           ``forward(x, batch, cache, state, residual) -> pending``
 * ``FeedForward``     ``forward(x, residual) -> pending``
 * ``Block``           ``forward(residual, batch, cache, state, pending) -> pending`` (where norms and sums sit)
@@ -61,10 +61,11 @@ class StateNeed:
 @dataclass(frozen=True)
 class Rotation:
     """Rotary position encoding as a mixer's kernels need it: the first ``dim`` elements of each
-    head are turned in pairs (j, j + dim/2) by ``position * inv_freq[j]``."""
+    head are turned in pairs (j, j + dim/2) by the step's angles, whose cosines and sines are the two
+    halves of a row of ``table``."""
 
     dim: int
-    inv_freq: Any  # float32 device tensor [dim / 2]
+    table: Any  # float32 device tensor [tokens of the step, dim]: cosines, then sines
 
 
 class Runtime:
@@ -107,7 +108,10 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    def rotation(self) -> Rotation | None:
+    def rotation(self, batch) -> Rotation | None:
+        """What the mixer turns q and k by in this step. Anything computed from the step's positions
+        alone belongs in ``batch.memo`` (a dict that lives as long as the step), under a key that names
+        the encoding's constants, so that layers with equal constants compute it once."""
         return None
 
 

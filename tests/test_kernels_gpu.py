@@ -191,16 +191,41 @@ def plain_rope(x, pos, inv_freq, rot):
     return out
 
 
+def test_rope_table(ops):
+    pos = torch.tensor([0, 1, 2, 77, 4095, 40000], dtype=torch.int32, device=DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, 48, 2).float() / 48))).to(DEV)
+    table = ops.rope_table(pos, inv_freq)
+    ang = (pos.float()[:, None] * inv_freq[None, :]).double()  # the angle itself is a float32 product
+    assert table.shape == (6, 48) and table.dtype == F32
+    close(table[:, :24], torch.cos(ang), 1e-6, "cosines")
+    close(table[:, 24:], torch.sin(ang), 1e-6, "sines")
+    assert torch.equal(table[0, :24], torch.ones(24, device=DEV)) and torch.equal(table[0, 24:], torch.zeros(24, device=DEV))
+
+
+# (tokens, layout of the slots): few tokens run the kernel with a wave per head, many the tiled one,
+# whose value store takes whole aligned runs of a page with one vector and everything else singly.
+QK_CASES = [(11, "scattered"), (150, "scattered"), (150, "runs"), (200, "shifted")]
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 1, 32, 32, 16), (3, 3, 48, 24, 8), (5, 5, 256, 256, 4), (16, 8, 128, 128, 16)])
-def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
-    t, pages, eps = 11, 9, 1e-5
+@pytest.mark.parametrize("t,layout", QK_CASES)
+@pytest.mark.parametrize("hq,hkv,d,rot,page", [(4, 2, 16, 16, 16), (6, 1, 32, 32, 16), (3, 3, 48, 24, 8), (5, 5, 256, 256, 4),
+                                               (16, 8, 128, 128, 16), (3, 1, 64, 64, 16), (2, 2, 128, 0, 8), (4, 2, 64, 32, 16)])
+def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page, t, layout):
+    pages, eps = (t + page - 1) // page + 9, 1e-5
     qkv = rand((t, (hq + 2 * hkv) * d), dtype, 16)
     qw, kw = rand((d,), dtype, 17) + 1, rand((d,), dtype, 18) + 1
-    pos = torch.tensor([0, 1, 2, 3, 40, 41, 700, 5, 6, 7, 4000], dtype=torch.int32, device=DEV)
-    perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(1))[:t]
+    pos = torch.tensor(([0, 1, 2, 3, 40, 41, 700, 5, 6, 7, 4000] * 20)[:t], dtype=torch.int32, device=DEV)
+    if layout == "scattered":
+        perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(1))[:t]
+    elif layout == "runs":  # consecutive slots from a page's start, as a prompt's portion has them
+        perm = torch.arange(t) + 2 * page
+    else:  # consecutive, but starting in the middle of a page and with a jump to another page
+        second = (93 // page + 3) * page + 5
+        perm = torch.cat([torch.arange(3, 3 + 90), torch.arange(second, second + t - 90)])
     slots = perm.to(torch.int32).to(DEV)
-    inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / max(rot, 1)))).to(DEV)
+    rope = ops.rope_table(pos, inv_freq) if rot else None
     kc = torch.full((pages, hkv, page, d), 7.0, dtype=dtype, device=DEV)
     vc = torch.full((pages, hkv, d, page), 7.0, dtype=dtype, device=DEV)  # values lie transposed within the page
     ref = qkv.double().view(t, hq + 2 * hkv, d)
@@ -209,10 +234,10 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
     def norm(x, w):
         return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
 
-    qn = plain_rope(norm(q, qw), pos, inv_freq, rot)
-    kn = plain_rope(norm(k, kw), pos, inv_freq, rot)
+    qn = plain_rope(norm(q, qw), pos, inv_freq, rot) if rot else norm(q, qw)
+    kn = plain_rope(norm(k, kw), pos, inv_freq, rot) if rot else norm(k, kw)
     work = qkv.clone()
-    ops.qk_norm_rope_store(work, pos, slots, qw, kw, eps, inv_freq, rot, kc, vc, hq, hkv, d)
+    ops.qk_norm_rope_store(work, slots, qw, kw, eps, rope, kc, vc, hq, hkv, d)
     tol = 2e-6 if dtype == F32 else 5e-3
     close(work.view(t, hq + 2 * hkv, d)[:, :hq], qn, tol, "q")
     sl = slots.long()
@@ -228,7 +253,7 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page):
     # the same from partial sums of qkv: queries come back in a tensor of their own
     parts = torch.stack([qkv.float() * 0.25, qkv.float() * 0.5, qkv.float() * 0.25])
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
-    q2 = ops.qk_norm_rope_store(ops.SplitSum(parts), pos, slots, qw, kw, eps, inv_freq, rot, kc2, vc2, hq, hkv, d, out_dtype=dtype)
+    q2 = ops.qk_norm_rope_store(ops.SplitSum(parts), slots, qw, kw, eps, rope, kc2, vc2, hq, hkv, d, out_dtype=dtype)
     assert q2.shape == (t, hq * d)
     close(q2.view(t, hq, d), qn, tol, "q from partial sums")
     close(kc2.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)[sl], kn, tol, "k from partial sums")
