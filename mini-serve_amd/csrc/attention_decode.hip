@@ -8,9 +8,11 @@
 // Both feed v_mfma_f32_16x16x32_bf16 straight from global memory with one vector load per lane:
 //   scores  S^T[token, query] : A operand = K rows (i = token), B operand = Q (j = query head of the group)
 //   output  O[query, d]       : A operand = P (i = query, k = token), B operand = V^T (j = d, k = token)
-// A lane of the score result holds 4 tokens of one query for each of two pages; the MFMA's k index
-// of the second product is mapped to tokens so that exactly these 8 values are the lane's P operand:
-// probabilities never move between lanes.
+// The two score products of a 32-token chunk take their key rows in an order chosen so that a lane
+// of the results holds 8 consecutive tokens of one page for one query (lane group g: page g / 2 of
+// the chunk, tokens 8 (g % 2) .. + 7; four from each product). The MFMA's k index of the second
+// product is mapped to tokens in the same way, so exactly these 8 values are the lane's P operand
+// (probabilities never move between lanes) and its V^T operand is one 16-byte load.
 //
 // Grid: (rows * Hkv, splits). A block of 4 waves takes a contiguous range of 32-token chunks; its
 // waves take chunks in turn and are merged in LDS. splits == 1 writes the result directly.
@@ -27,7 +29,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 template <int D>
 struct DecodeTile {
   bf16x8 ka[D / 32], kb[D / 32];
-  bf16x4 va[D / 16], vb[D / 16];
+  bf16x8 v[D / 16];
 };
 
 template <int D>
@@ -85,21 +87,20 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     const int p0 = max(p0n, 0);  // a page behind the window was given back: its tokens are masked below
     const int p1 = max(p1n, 0);
     fetch_ids(c + 4);
-    const bf16* k0 = kc + (((size_t)p0 * Hkv + kvh) * PAGE + r) * D + g * 8;
-    const bf16* k1 = kc + (((size_t)p1 * Hkv + kvh) * PAGE + r) * D + g * 8;
+    // Key rows: lane r feeds row r of both products. Product a takes tokens 0-3 and 8-11 of each page,
+    // product b tokens 4-7 and 12-15 (rows 0-7 from the chunk's first page, 8-15 from its second).
+    const int kp = r < 8 ? p0 : p1;
+    const int kt = (r % 4) + 8 * ((r / 4) % 2);
+    const bf16* k0 = kc + (((size_t)kp * Hkv + kvh) * PAGE + kt) * D + g * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       t.ka[kk] = *reinterpret_cast<const bf16x8*>(k0 + kk * 32);
-      t.kb[kk] = *reinterpret_cast<const bf16x8*>(k1 + kk * 32);
+      t.kb[kk] = *reinterpret_cast<const bf16x8*>(k0 + 4 * D + kk * 32);
     }
-    // V^T operand: element d = db * 16 + r, tokens 4 g .. 4 g + 3 of each page.
-    const bf16* v0 = vc + (((size_t)p0 * Hkv + kvh) * D + r) * PAGE + g * 4;
-    const bf16* v1 = vc + (((size_t)p1 * Hkv + kvh) * D + r) * PAGE + g * 4;
+    // V^T operand: element d = db * 16 + r, tokens 8 (g % 2) .. + 7 of page g / 2.
+    const bf16* v0 = vc + (((size_t)(g < 2 ? p0 : p1) * Hkv + kvh) * D + r) * PAGE + (g % 2) * 8;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      t.va[db] = *reinterpret_cast<const bf16x4*>(v0 + (size_t)db * 16 * PAGE);
-      t.vb[db] = *reinterpret_cast<const bf16x4*>(v1 + (size_t)db * 16 * PAGE);
-    }
+    for (int db = 0; db < DB; ++db) t.v[db] = *reinterpret_cast<const bf16x8*>(v0 + (size_t)db * 16 * PAGE);
   };
   auto multiply = [&](const DecodeTile<D>& t, int c) {
     const int t0 = lo_al + c * CHUNK;
@@ -109,12 +110,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
       s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.ka[kk], qf[kk], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.kb[kk], qf[kk], s1, 0, 0, 0);
     }
-    // This lane: tokens t0 + 4 g + i (s0) and t0 + 16 + 4 g + i (s1) of query r.
+    // This lane: tokens tl + i (s0) and tl + 4 + i (s1) of query r, tl = t0 + 16 (g / 2) + 8 (g % 2).
+    const int tl = t0 + 8 * g;
     float sc[8];
     float m_new = m_run;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int ta = t0 + 4 * g + i, tb = ta + PAGE;
+      const int ta = tl + i, tb = ta + 4;
       sc[i] = (ta >= lo && ta < kv_len) ? s0[i] * scale : -INFINITY;
       sc[4 + i] = (tb >= lo && tb < kv_len) ? s1[i] * scale : -INFINITY;
       m_new = fmaxf(m_new, fmaxf(sc[i], sc[4 + i]));
@@ -144,13 +146,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     for (int db = 0; db < DB; ++db) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[db][i] *= cq[i];
-      bf16x8 vf;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        vf[i] = t.va[db][i];
-        vf[4 + i] = t.vb[db][i];
-      }
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, t.v[db], o[db], 0, 0, 0);
     }
   };
   {

@@ -43,7 +43,8 @@ _SIGNATURES = {
     "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
                                   _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
-    "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
+    "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
+    "ms_sample_scratch_bytes": [_c_int],
 }
 
 
@@ -479,6 +480,11 @@ def sample_rows(logits, temperature=None, top_p=None, seed=None, counter=None) -
             if v.shape[0] != rows:
                 raise ValueError("one sampling parameter per row is needed")
     out = torch.empty((rows,), dtype=I32, device=logits.device)
-    _check(library().ms_sample_rows(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
-                                    _ptr(counter), out.data_ptr(), _stream()), "sample_rows")
+    lib = library()
+    need = lib.ms_sample_scratch_bytes(rows)
+    if need < 0:
+        raise ValueError(f"sample_rows: {rows} rows are more than one call takes")
+    scratch = torch.empty((need,), dtype=torch.uint8, device=logits.device)
+    _check(lib.ms_sample_rows(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
+                              _ptr(counter), scratch.data_ptr(), out.data_ptr(), _stream()), "sample_rows")
     return out
