@@ -203,37 +203,40 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
   }
 }
 
-// Reduction of the splits in ascending order: grid (rows, Hq), D threads. Loads go out eight splits
-// at a time so that their latencies overlap.
+// Reduction of the splits in ascending order: grid (rows, Hq), D threads. Loads go out 32 splits at
+// a time (all of them, for most shapes), so that their latencies overlap; the order of the sums is
+// the order of the splits whatever the batching.
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
                                                                 const int* __restrict__ tokens, bf16* __restrict__ out,
                                                                 int Hq, int splits) {
+  constexpr int NB = 32;
   const int b = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const size_t base = ((size_t)b * Hq + head) * splits;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
   float M = -INFINITY;
-  for (int s0 = 0; s0 < splits; s0 += 8) {
-    float m[8];
+  for (int s0 = 0; s0 < splits; s0 += NB) {
+    float m[NB];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) m[u] = s0 + u < splits ? part_ml[(base + s0 + u) * 2] : -INFINITY;
+    for (int u = 0; u < NB; ++u) m[u] = s0 + u < splits ? ml[s0 + u].x : -INFINITY;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) M = fmaxf(M, m[u]);
+    for (int u = 0; u < NB; ++u) M = fmaxf(M, m[u]);
   }
   float L = 0.f, O = 0.f;
-  for (int s0 = 0; s0 < splits; s0 += 8) {
-    float m[8], l[8], o[8];
+  for (int s0 = 0; s0 < splits; s0 += NB) {
+    float2 q[NB];
+    float o[NB];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < NB; ++u) {
       const bool in = s0 + u < splits;
-      m[u] = in ? part_ml[(base + s0 + u) * 2] : -INFINITY;
-      l[u] = in ? part_ml[(base + s0 + u) * 2 + 1] : 0.f;
+      q[u] = in ? ml[s0 + u] : make_float2(-INFINITY, 0.f);
       o[u] = in ? part_o[(base + s0 + u) * D + d] : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const float f = m[u] == -INFINITY ? 0.f : expf(m[u] - M);  // an empty or absent split adds nothing
-      L += l[u] * f;
+    for (int u = 0; u < NB; ++u) {
+      const float f = q[u].x == -INFINITY ? 0.f : expf(q[u].x - M);  // an empty or absent split adds nothing
+      L += q[u].y * f;
       O += o[u] * f;
     }
   }

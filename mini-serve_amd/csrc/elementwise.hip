@@ -80,6 +80,68 @@ __global__ __launch_bounds__(NT) void rmsnorm_kernel(float* __restrict__ x, cons
   }
 }
 
+// The same for few rows of a width that is a multiple of 4 and at most 8 NT, bfloat16 output: NT
+// threads per row, a thread owns up to two groups of 4 consecutive elements and moves them as vectors;
+// the partial sums of 8 splits are fetched at a time. Sums per element in ascending split order, as
+// in the kernel above.
+template <typename TW, int NT>
+__global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x, const TW* __restrict__ w,
+                                                            bf16* __restrict__ y, const int* __restrict__ rows, int width,
+                                                            float eps, const float* __restrict__ parts, int splits,
+                                                            size_t split_stride) {
+  __shared__ float red[NT / WAVE];
+  const int r = blockIdx.x;
+  const size_t row = rows ? rows[r] : r;
+  float* src = x + row * width;
+  const bool in_place = parts != nullptr && rows == nullptr;
+  float4 kept[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = (threadIdx.x + j * NT) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < width) {
+      v = *reinterpret_cast<const float4*>(src + i);
+      if (parts != nullptr) {
+        const float* p = parts + row * width + i;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+          float4 t[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const bool in = s0 + u < splits;
+            t[u] = *reinterpret_cast<const float4*>(p + (size_t)(in ? s0 + u : 0) * split_stride);
+            if (!in) t[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            acc.x += t[u].x; acc.y += t[u].y; acc.z += t[u].z; acc.w += t[u].w;
+          }
+        }
+        v.x += acc.x; v.y += acc.y; v.z += acc.z; v.w += acc.w;
+        if (in_place) *reinterpret_cast<float4*>(src + i) = v;
+      }
+    }
+    kept[j] = v;
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float rstd = rsqrtf(ss / (float)width + eps);
+  bf16* dst = y + (size_t)r * width;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = (threadIdx.x + j * NT) * 4;
+    if (i < width) {
+      union { uint2 u; bf16 e[4]; } o;
+      o.e[0] = from_f32<bf16>(kept[j].x * rstd * to_f32(w[i]));
+      o.e[1] = from_f32<bf16>(kept[j].y * rstd * to_f32(w[i + 1]));
+      o.e[2] = from_f32<bf16>(kept[j].z * rstd * to_f32(w[i + 2]));
+      o.e[3] = from_f32<bf16>(kept[j].w * rstd * to_f32(w[i + 3]));
+      *reinterpret_cast<uint2*>(dst + i) = o.u;
+    }
+  }
+}
+
 extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y_is_bf16, const int* rows, int n_rows,
                           int width, float eps, const float* parts, int splits, long long split_stride, hipStream_t st) {
   if (n_rows <= 0) return MS_OK;
@@ -87,6 +149,18 @@ extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y
   // float32 output keeps one block shape for every batch, so that its sums are formed in one order
   // whatever the batch; bfloat16 output takes the wide block for few rows.
   const bool wide = y_is_bf16 && n_rows <= 256;
+  if (wide && width % 4 == 0 && width <= 8192 && (parts == nullptr || split_stride % 4 == 0)) {
+#define LAUNCH_VEC(TW)                                                                                                  \
+  if (width <= 2048)                                                                                                    \
+    rmsnorm_vec4_kernel<TW, 256><<<n_rows, 256, 0, st>>>(x, (const TW*)w, (bf16*)y, rows, width, eps, parts, splits,    \
+                                                          (size_t)split_stride);                                        \
+  else                                                                                                                  \
+    rmsnorm_vec4_kernel<TW, 1024><<<n_rows, 1024, 0, st>>>(x, (const TW*)w, (bf16*)y, rows, width, eps, parts, splits,  \
+                                                            (size_t)split_stride)
+    if (w_is_bf16) { LAUNCH_VEC(bf16); } else { LAUNCH_VEC(float); }
+#undef LAUNCH_VEC
+    return launch_status();
+  }
 #define LAUNCH(TW, TO)                                                                                                  \
   if (wide)                                                                                                             \
     rmsnorm_kernel<TW, TO, 1024, 4><<<n_rows, 1024, 0, st>>>(x, (const TW*)w, (TO*)y, rows, width, eps, parts, splits,  \
@@ -332,11 +406,21 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_tile_kernel(
   if (parts != nullptr) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = 0.f;
-    for (int s = 0; s < splits; ++s) {  // ascending split order; the two loads of a split go out together
-      const float4 a = *reinterpret_cast<const float4*>(parts + (size_t)s * split_stride + at);
-      const float4 b = *reinterpret_cast<const float4*>(parts + (size_t)s * split_stride + at + 4);
-      x[0] += a.x; x[1] += a.y; x[2] += a.z; x[3] += a.w;
-      x[4] += b.x; x[5] += b.y; x[6] += b.z; x[7] += b.w;
+    for (int s0 = 0; s0 < splits; s0 += 4) {  // ascending split order; the loads of four splits go out together
+      float4 a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool in = s0 + u < splits;
+        const float* src = parts + (size_t)(in ? s0 + u : 0) * split_stride + at;
+        a[u] = *reinterpret_cast<const float4*>(src);
+        b[u] = *reinterpret_cast<const float4*>(src + 4);
+        if (!in) a[u] = b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        x[0] += a[u].x; x[1] += a[u].y; x[2] += a[u].z; x[3] += a[u].w;
+        x[4] += b[u].x; x[5] += b[u].y; x[6] += b[u].z; x[7] += b[u].w;
+      }
     }
   } else {
     Vec8<T> v;

@@ -314,7 +314,9 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
 // its loads at once, unless that would make more waves than the chip holds a few times over (then
 // slices of several whole slabs). With up to 16 rows the partial sums are small beside the weights
-// and 32768 waves are allowed; above that 8192. The count depends on M only through that class.
+// and 32768 waves are allowed; above that 8192. At most 16 splits: the kernel that sums them up reads
+// every one. The count depends on M only through that class.
+#define SMALL_MAX_SPLITS 16
 static int small_slabs_per_split(int M, int N, int K) {
   const int slabs = (K + SMALL_SLAB - 1) / SMALL_SLAB;
   const int row_blocks = (N + 15) / 16;
@@ -322,6 +324,7 @@ static int small_slabs_per_split(int M, int N, int K) {
   int s = slabs;
   const int most = waves / row_blocks > 0 ? waves / row_blocks : 1;
   if (s > most) s = most;
+  if (s > SMALL_MAX_SPLITS) s = SMALL_MAX_SPLITS;
   return (slabs + s - 1) / s;
 }
 

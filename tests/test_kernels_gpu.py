@@ -63,6 +63,28 @@ def test_rmsnorm(ops, width, w_dtype, out_dtype):
     close(got, want[rows.long()], 1e-6 if out_dtype == F32 else 5e-3, "rmsnorm rows")
 
 
+@pytest.mark.parametrize("width,splits", [(96, 3), (1000, 11), (1024, 8), (5120, 16), (4098, 2)])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_rmsnorm_adds_partial_sums(ops, width, splits, out_dtype):
+    """Every shape of the norm kernels (vector and scalar, one or several groups per thread, a number
+    of splits that is no multiple of the load batch) adds the partial sums in full, with and without a
+    row list."""
+    m, eps = 5, 1e-6
+    x = rand((m, width), F32, 60, 2.0)
+    parts = rand((splits, m, width), F32, 61)
+    w = rand((width,), BF16, 62) + 1
+    full = x.double() + parts.double().sum(0)
+    want = full / torch.sqrt((full * full).mean(-1, keepdim=True) + eps) * w.double()
+    tol = 1e-5 if out_dtype == F32 else 5e-3
+    x1 = x.clone()
+    close(ops.rmsnorm(x1, w, eps, out_dtype, add=ops.SplitSum(parts)), want, tol, "all rows")
+    close(x1, full, 1e-6, "stream brought up to date")
+    x2 = x.clone()
+    rows = torch.tensor([4, 1, 1], dtype=torch.int32, device=DEV)
+    close(ops.rmsnorm(x2, w, eps, out_dtype, rows, add=ops.SplitSum(parts)), want[rows.long()], tol, "row list")
+    assert torch.equal(x2, x)
+
+
 def test_rmsnorm_eps_enters(ops):
     x = rand((2, 64), F32, 4, 1e-3)
     w = torch.ones(64, device=DEV)
