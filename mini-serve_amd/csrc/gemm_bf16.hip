@@ -1,8 +1,11 @@
 // bfloat16 matrix products C[M, N] = X[M, K] * W[N, K]^T on the gfx950 matrix cores
-// (v_mfma_f32_16x16x32_bf16, float32 accumulation), in two shapes:
+// (v_mfma_f32_16x16x32_bf16, float32 accumulation), in three shapes:
 //
-//  * tile kernel   (prefill, M large): BM x BN macro-tiles staged through LDS in K-slabs of 64 with a
-//                  register prefetch of the next slab; 4 waves in a 2 x 2 grid of wave tiles.
+//  * tile kernel, slabs straight into LDS (prefill, M large, K a multiple of 64): 128 x 128 macro-tiles,
+//                  K-slabs of 64 loaded by global_load_lds into a ring of two stages with a bank
+//                  swizzle, one barrier per slab, two blocks per CU; 4 waves in a 2 x 2 grid of wave tiles.
+//  * tile kernel, slabs through registers (any K and alignment, or few tiles): BM x BN macro-tiles
+//                  staged through LDS in K-slabs of 64 with a register prefetch of the next slab.
 //  * small-M kernel (decode, M <= 64): pure weight streaming. A wave owns 16 weight rows and a slice
 //                  of K, with 32-byte loads per lane; K is split over the grid into partial sums.
 //
@@ -100,7 +103,19 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(const bf16* __re
     for (int j = 0; j < FM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   Chunk xr[XCH], wr[WCH];
+  // A tile that lies wholly inside both matrices loads its slabs without any test (all loads of a
+  // slab go out back to back); edge tiles and the last, shorter slab take the checked loads.
+  const bool interior = vecx && vecw && m0 + BM <= M && n0 + BN <= N;
+  const bf16* xg = X + (size_t)(m0 + tid / (BK / 8)) * ldx + (tid % (BK / 8)) * 8;
+  const bf16* wg = W + (size_t)(n0 + tid / (BK / 8)) * Kfull + (tid % (BK / 8)) * 8;
   auto fetch = [&](int k0) __attribute__((always_inline)) {
+    if (interior && k0 + BK <= K) {
+#pragma unroll
+      for (int i = 0; i < XCH; ++i) xr[i].u = *reinterpret_cast<const uint4*>(xg + (size_t)i * (256 / (BK / 8)) * ldx + k0);
+#pragma unroll
+      for (int i = 0; i < WCH; ++i) wr[i].u = *reinterpret_cast<const uint4*>(wg + (size_t)i * (256 / (BK / 8)) * Kfull + k0);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       const int c = tid + i * 256;
@@ -149,6 +164,117 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(const bf16* __re
     if (more) {
       stash();
       __syncthreads();
+    }
+  }
+
+  const bool vec_store = (ldc % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j)
+      store4(C, mode, m0 + wm + j * 16 + r, n0 + wn + i * 16 + g * 4, M, N, ldc, acc[i][j], vec_store);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tile kernel with slabs loaded straight into LDS (global_load_lds, 16 bytes per lane): no staging
+// registers and no LDS store instructions, STAGES slabs of 64 k in a ring, one barrier per slab. A load
+// instruction of a wave fills 1 KB of LDS in lane order, that is 8 rows of 128 bytes; which 16-byte
+// chunk of its row a lane fetches is chosen so that chunk c of tile row R lands in slot
+// c ^ ((R >> 1) & 7) of the row: fragment reads (16 rows, one chunk column) then touch every bank
+// once. Rows beyond M or N are read from the last valid row (their results are never stored); K must
+// be a multiple of 64 and rows 16-byte aligned, which the caller checks.
+
+// Wait until at most N of this wave's vector-memory loads are in flight (expcnt and lgkmcnt are left alone).
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
+__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                               void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
+                                                               int ldx, int ldc, int k_per, size_t c_split_stride) {
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int FM = WM / 16, FN = WN / 16;
+  constexpr int ROW_BYTES = KS * 2;           // a tile row: KS k of bf16
+  constexpr int CPR = KS / 8;                 // 16-byte chunks per row
+  constexpr int RPI = 1024 / ROW_BYTES;       // rows a load instruction of a wave fills
+  constexpr int XI = BM / (4 * RPI), WI = BN / (4 * RPI);  // load instructions per wave and slab
+  constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // STAGES * STAGE_BYTES
+
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
+  const int k_lo = blockIdx.z * k_per;
+  const int K = min(Kfull, k_lo + k_per);
+  const int slabs = (K - k_lo) / KS;
+  void* C = mode == 1 ? (void*)((float*)Cbase + blockIdx.z * c_split_stride) : Cbase;
+
+  // Load side: instruction j of this wave fills tile rows (wave * XI + j) * 8 .. + 7.
+  const int lrow = lane / CPR, lslot = lane % CPR;
+  const bf16* xsrc[XI];
+  const bf16* wsrc[WI];
+#pragma unroll
+  for (int j = 0; j < XI; ++j) {
+    const int R = (wave * XI + j) * RPI + lrow;
+    xsrc[j] = X + (size_t)min(m0 + R, M - 1) * ldx + k_lo + ((lslot ^ ((R >> 1) & (CPR - 1))) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < WI; ++j) {
+    const int R = (wave * WI + j) * RPI + lrow;
+    wsrc[j] = W + (size_t)min(n0 + R, N - 1) * Kfull + k_lo + ((lslot ^ ((R >> 1) & (CPR - 1))) * 8);
+  }
+  auto issue = [&](int slab) __attribute__((always_inline)) {
+    unsigned char* stage = lds + (slab % STAGES) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < XI; ++j)
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(xsrc[j] + (size_t)slab * KS),
+                                       (void __attribute__((address_space(3)))*)(stage + (wave * XI + j) * 1024),
+                                       16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < WI; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (const void __attribute__((address_space(1)))*)(wsrc[j] + (size_t)slab * KS),
+          (void __attribute__((address_space(3)))*)(stage + BM * ROW_BYTES + (wave * WI + j) * 1024), 16, 0, 0);
+  };
+
+  floatx4 acc[FN][FM];
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // Read side: the rows of a fragment are base + r with base a multiple of 16, so the slot of chunk c
+  // is c ^ (r >> 1) for every fragment.
+  const int sw = (r >> 1) & (CPR - 1);
+  const int x_off = (wm + r) * ROW_BYTES, w_off = BM * ROW_BYTES + (wn + r) * ROW_BYTES;
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < slabs) issue(s);
+  for (int k = 0; k < slabs; ++k) {
+    // Slab k must have landed; the STAGES - 2 slabs after it may stay in flight (near the end there
+    // are fewer of them: then everything is waited for).
+    if (k + STAGES - 2 < slabs) wait_loads<(XI + WI) * (STAGES - 2)>();
+    else wait_loads<0>();
+    __syncthreads();  // slab k has landed for every wave, and every wave is done with slab k - 1
+    if (k + STAGES - 1 < slabs) issue(k + STAGES - 1);
+    const unsigned char* stage = lds + (k % STAGES) * STAGE_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < CPR; kk += 4) {  // chunk columns kk + g
+      const int slot = ((kk + g) ^ sw) * 16;
+      bf16x8 wf[FN], xf[FM];
+#pragma unroll
+      for (int i = 0; i < FN; ++i) wf[i] = *reinterpret_cast<const bf16x8*>(stage + w_off + i * 16 * ROW_BYTES + slot);
+#pragma unroll
+      for (int j = 0; j < FM; ++j) xf[j] = *reinterpret_cast<const bf16x8*>(stage + x_off + j * 16 * ROW_BYTES + slot);
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[j], acc[i][j], 0, 0, 0);
     }
   }
 
@@ -370,6 +496,23 @@ extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
   return s;
 }
 
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
+static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
+                      size_t stride, int splits, hipStream_t st) {
+  constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
+  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits);
+  if (grid.y > 65535) return MS_BAD_ARG;
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<grid, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
+  return launch_status();
+}
+
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
 // splits > 1 (mode 1 only): C holds splits * M * N floats of partial sums, slice after slice.
 extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,
@@ -385,6 +528,11 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   const size_t stride = (size_t)M * N;
   // Large tiles when they still give every CU work; small tiles otherwise.
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128) * splits;
+  // Whole 64-k slabs and 16-byte aligned rows: the kernel whose slabs go straight into LDS. Of the
+  // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
+  // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
+  if (K % BK == 0 && ldx % 8 == 0 && big >= 256)
+    return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
   if (big >= 256) {
     dim3 grid((N + 127) / 128, (M + 127) / 128, splits);
     if (grid.y > 65535) return MS_BAD_ARG;

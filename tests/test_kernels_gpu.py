@@ -137,6 +137,21 @@ def test_gemm_bf16(ops, m, n, k):
     close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
 
 
+@pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024)])
+def test_gemm_bf16_large_tiles(ops, m, n, k):
+    """Shapes with at least 256 tiles of 128 x 128 and K a multiple of 64 take the kernel whose slabs go
+    straight into LDS: edge tiles in both directions (rows past the end are read from the last valid
+    row and never stored), one slab, an odd number of slabs."""
+    x, w = rand((m, k), BF16, 14), rand((n, k), BF16, 15)
+    want = x.double() @ w.double().T
+    close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
+    close(ops.linear(x, w, out_dtype=BF16), want, 5e-3, "gemm bf16 -> bf16")
+    acc = rand((m, n), F32, 16)
+    before = acc.clone()
+    ops.linear(x, w, accumulate_into=acc)
+    close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 40, 64])
 def test_pending_sums_feed_their_consumers(ops, m):
     """The small-M product may leave partial sums for the next kernel to add: every consumer of such
