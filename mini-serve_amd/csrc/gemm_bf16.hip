@@ -437,6 +437,23 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
   return launch_status();
 }
 
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
+static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
+                      size_t stride, int splits, hipStream_t st) {
+  constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
+  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits);
+  if (grid.y > 65535) return MS_BAD_ARG;
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<grid, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
+  return launch_status();
+}
+
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
 // its loads at once, unless that would make more waves than the chip holds a few times over (then
 // slices of several whole slabs). With up to 16 rows the partial sums are small beside the weights
@@ -454,7 +471,27 @@ static int small_slabs_per_split(int M, int N, int K) {
   return (slabs + s - 1) / s;
 }
 
+// 16 < M <= 64 and K a multiple of 64: the product runs as 64 x 64 tiles of the kernel whose slabs go
+// straight into LDS (it streams the weights faster than the four-wave small-M kernel: 2.9 -> 4.4 TB/s
+// at the 8B shapes), with K split so that about 768 blocks are in the grid, at most 16 splits and at
+// least two slabs per split.
+static bool small_runs_as_tiles(int M, int K) { return M > 16 && K % BK == 0; }
+
+static int tile_slabs_per_split(int N, int K) {
+  const int slabs = K / BK;
+  const int cols = (N + 63) / 64;
+  int s = (768 + cols - 1) / cols;
+  if (s > SMALL_MAX_SPLITS) s = SMALL_MAX_SPLITS;
+  if (s > slabs / 2) s = slabs / 2;
+  if (s < 1) s = 1;
+  return (slabs + s - 1) / s;
+}
+
 extern "C" int ms_gemm_bf16_small_splits(int M, int N, int K) {
+  if (small_runs_as_tiles(M, K)) {
+    const int per = tile_slabs_per_split(N, K);
+    return (K / BK + per - 1) / per;
+  }
   const int slabs = (K + SMALL_SLAB - 1) / SMALL_SLAB;
   const int per = small_slabs_per_split(M, N, K);
   return (slabs + per - 1) / per;  // no empty split
@@ -468,6 +505,18 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64 || K <= 0 || ldx < K || partials == nullptr) return MS_BAD_ARG;
   const int splits = ms_gemm_bf16_small_splits(M, N, K);
+  if (small_runs_as_tiles(M, K) && ldx % 8 == 0) {
+    const int k_per = tile_slabs_per_split(N, K) * BK;
+    const int rc = launch_dma<64, 64, BK, 2, 4>((const bf16*)X, (const bf16*)W, partials, 1, M, N, K, ldx, N, k_per,
+                                                 (size_t)M * N, splits, st);
+    if (rc != MS_OK) return rc;
+    if (reduce) {
+      if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
+      splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);
+    }
+    return launch_status();
+  }
+  if (small_runs_as_tiles(M, K)) return MS_BAD_ARG;  // the split count was made for the tile kernel
   const int per = small_slabs_per_split(M, N, K) * (SMALL_SLAB / 64);
   const long wave_blocks = (long)((N + 15) / 16) * splits, wide_blocks = (long)((N + 63) / 64) * splits;
   if (wave_blocks > 0x7fffffffL) return MS_BAD_ARG;
@@ -496,23 +545,6 @@ extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
   return s;
 }
 
-template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
-static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
-                      size_t stride, int splits, hipStream_t st) {
-  constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
-  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
-  if (!ready) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-      return MS_LAUNCH_FAILED;
-    ready = true;
-  }
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits);
-  if (grid.y > 65535) return MS_BAD_ARG;
-  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<grid, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
-  return launch_status();
-}
-
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
 // splits > 1 (mode 1 only): C holds splits * M * N floats of partial sums, slice after slice.
 extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,
@@ -531,8 +563,10 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   // Whole 64-k slabs and 16-byte aligned rows: the kernel whose slabs go straight into LDS. Of the
   // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
   // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
-  if (K % BK == 0 && ldx % 8 == 0 && big >= 256)
-    return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+  if (K % BK == 0 && ldx % 8 == 0) {
+    if (big >= 256) return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    return launch_dma<64, 64, BK, 2, 4>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+  }
   if (big >= 256) {
     dim3 grid((N + 127) / 128, (M + 127) / 128, splits);
     if (grid.y > 65535) return MS_BAD_ARG;

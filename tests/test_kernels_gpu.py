@@ -162,8 +162,9 @@ def test_pending_sums_feed_their_consumers(ops, m):
     s = ops.linear(x, w, out_dtype=BF16, defer=True)
     assert isinstance(s, ops.SplitSum) and s.splits > 1 and s.shape == (m, n)
     close(s.parts.sum(0), want, 1e-5, "partial sums")
-    # the number of splits depends on the matrix alone, not on the rows
-    assert ops.linear(x[:1].contiguous(), w, out_dtype=BF16, defer=True).splits == s.splits
+    # the number of splits depends on the matrix and on whether there are more than 16 rows, not on the rows themselves
+    other = x[:1] if m <= 16 else torch.cat([x, x])[:17]
+    assert ops.linear(other.contiguous(), w, out_dtype=BF16, defer=True).splits == s.splits
     # residual stream: norm with the pending sum added first, rows or all
     resid = rand((m, n), F32, 52)
     nw = rand((n,), BF16, 53) + 1
