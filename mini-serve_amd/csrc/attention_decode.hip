@@ -7,7 +7,7 @@
 //                                                head element are contiguous
 // Both feed v_mfma_f32_16x16x32_bf16 straight from global memory with one vector load per lane:
 //   scores  S^T[token, query] : A operand = K rows (i = token), B operand = Q (j = query head of the group)
-//   output  O[query, d]       : A operand = P (i = query, k = token), B operand = V^T (j = d, k = token)
+//   output  O^T[d, query]     : A operand = V^T (i = d, k = token), B operand = P (j = query, k = token)
 // The two score products of a 32-token chunk take their key rows in an order chosen so that a lane
 // of the results holds 8 consecutive tokens of one page for one query (lane group g: page g / 2 of
 // the chunk, tokens 8 (g % 2) .. + 7; four from each product). The MFMA's k index of the second
@@ -121,8 +121,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
       sc[4 + i] = (tb >= lo && tb < kv_len) ? s1[i] * scale : -INFINITY;
       m_new = fmaxf(m_new, fmaxf(sc[i], sc[4 + i]));
     }
-    m_new = fmaxf(m_new, __shfl_xor(m_new, 16, WAVE));
-    m_new = fmaxf(m_new, __shfl_xor(m_new, 32, WAVE));
+    m_new = rows4_max(m_new);
     // A chunk that holds no visible token at all cannot occur: chunks start at the window's first
     // token's chunk and end at the last token's.
     float psum = 0.f;
@@ -133,20 +132,16 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
       psum += p;
       pf[i] = static_cast<bf16>(p);
     }
-    psum += __shfl_xor(psum, 16, WAVE);
-    psum += __shfl_xor(psum, 32, WAVE);
+    psum = rows4_sum(psum);
     const float corr = expf(m_run - m_new);
     l_run = l_run * corr + psum;
     m_run = m_new;
-    // Output rows are queries 4 g + i: fetch their correction from the lanes that own those queries.
-    float cq[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) cq[i] = __shfl(corr, 4 * g + i, WAVE);
+    // O^T[d, query]: a lane's output values are all of its own query r.
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[db][i] *= cq[i];
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, t.v[db], o[db], 0, 0, 0);
+      for (int i = 0; i < 4; ++i) o[db][i] *= corr;
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v[db], pf, o[db], 0, 0, 0);
     }
   };
   {
@@ -175,7 +170,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) so[wave][4 * g + i][db * 16 + r] = o[db][i];
+    for (int i = 0; i < 4; ++i) so[wave][r][db * 16 + 4 * g + i] = o[db][i];
   __syncthreads();
   for (int e = tid; e < G * D; e += 256) {
     const int qh = e / D, d = e % D;

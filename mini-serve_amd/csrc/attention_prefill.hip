@@ -4,11 +4,17 @@
 //
 // Work item = (tile of consecutive new tokens of one sequence, KV head). A block owns 64 NQ query
 // rows = tokens x the G query heads of the group (row = token * G + head), so K and V are read once
-// for the whole group. Keys are walked in tiles of 64 tokens staged in LDS: K as [token][D], V as
-// [D][token] (it already lies transposed within each page); page ids are fetched one tile ahead of
-// the tile's loads, the loads one tile ahead of the products. Operand roles as in the decode kernel:
-//   S^T[token, row] : A = K tile (i = token),  B = Q (j = row)      -> a lane holds 4 tokens of one row
-//   O[row, d]       : A = P (i = row, k = token), B = V^T (j = d)   -> those same values are its P operand
+// for the whole group. Keys are walked in tiles of 64 tokens held in LDS: K as [token][D], V as
+// [D][token] (it already lies transposed within each page). The tiles go straight from the cache pages
+// into a ring of LDS stages (global_load_lds, 16 bytes per lane, no staging registers and no LDS
+// stores), each row's 16-byte chunks permuted so that the fragment reads touch every bank once; page
+// ids are fetched one tile ahead of the tile's loads, the loads STAGES - 1 tiles ahead of the
+// products, and there is one barrier per tile. Operand roles as in the decode kernel:
+//   S^T[token, row] : A = K tile (i = token),  B = Q (j = row)
+//   O^T[d, row]     : A = V^T (i = d, k = token), B = P (j = row)   -> a lane's outputs are of its own row,
+//                                                                      whose maximum and sum it holds
+// The key rows of the two score products of a 32-key pair are taken in an order that leaves a lane
+// with 8 consecutive keys of one page: exactly its P operand, and its V^T operand is one 16-byte read.
 // Waves: 4 row groups of 16 NQ rows, times KSPLIT key groups. With KSPLIT == 2 two waves share a row
 // group and each takes half of every key tile (keeping its own running maximum, sum and output,
 // merged once at the end): a prompt of a few thousand tokens has too few tiles to fill the chip, and
@@ -35,64 +41,45 @@ __device__ __forceinline__ i32x4 tile_pages(const int* __restrict__ table, int t
   return *reinterpret_cast<const i32x4*>(table + idx);
 }
 
-// 16-byte chunks of a tile of TK keys, K [TK tokens][D] and V^T [D][TK tokens], spread over NT threads.
-// A page holds 2 D chunks of K and as many of V^T; chunk c = tid + NT i lies in page c / (2 D) of the
-// tile for both. Pages wholly past the last key (or given back behind a window) are replaced by a
-// valid page: their keys are masked.
-template <int D, int NT>
-__device__ __forceinline__ void fetch_tile(u32x4 (&kreg)[TK * (D / 8) / NT], u32x4 (&vreg)[TK * (D / 8) / NT],
-                                           const bf16* __restrict__ kc, const bf16* __restrict__ vc, i32x4 pages, int t0,
-                                           int last_pos, int Hkv, int kvh, int tid) {
-  constexpr int PP = NT / (2 * D);  // pages one pass of the block's threads covers
-  static_assert(PP >= 1 && (TK / PAGE) % PP == 0, "head size and block size");
-  const int t_eff = min(t0, (last_pos / TK) * TK);
-  const int sub = tid / (2 * D), within = tid % (2 * D);
-#pragma unroll
-  for (int i = 0; i < (TK / PAGE) / PP; ++i) {
-    int page = pages[i * PP];
-#pragma unroll
-    for (int k = 1; k < PP; ++k)
-      if (sub == k) page = pages[i * PP + k];
-    if (t_eff + (i * PP + sub) * PAGE > last_pos) page = pages[0];
-    page = max(page, 0);
-    kreg[i] = *reinterpret_cast<const u32x4*>(kc + (((size_t)page * Hkv + kvh) * PAGE + within / (D / 8)) * D + (within % (D / 8)) * 8);
-    vreg[i] = *reinterpret_cast<const u32x4*>(vc + (((size_t)page * Hkv + kvh) * D + within / 2) * PAGE + (within % 2) * 8);
-  }
+// Wait until at most N of this wave's vector-memory loads are in flight (expcnt and lgkmcnt are left alone).
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int D, int NT>
-__device__ __forceinline__ void stash_tile(const u32x4 (&kreg)[TK * (D / 8) / NT], const u32x4 (&vreg)[TK * (D / 8) / NT],
-                                           bf16* ks, bf16* vs, int tid) {
-  constexpr int KS = D + 8, VS = TK + 8;
-#pragma unroll
-  for (int i = 0; i < TK * (D / 8) / NT; ++i) {
-    const int c = tid + i * NT;
-    *reinterpret_cast<u32x4*>(&ks[(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = kreg[i];
-    const int pi = c / (2 * D), rem = c % (2 * D);
-    *reinterpret_cast<u32x4*>(&vs[(rem / 2) * VS + pi * PAGE + (rem % 2) * 8]) = vreg[i];
-  }
+// v[i] by three selects (no branch): i differs between the lanes of a wave.
+__device__ __forceinline__ int pick(i32x4 v, int i) {
+  int p = v[0];
+  p = i == 1 ? v[1] : p;
+  p = i == 2 ? v[2] : p;
+  p = i == 3 ? v[3] : p;
+  return p;
 }
 
-template <int D, int NQ, int KSPLIT>
-__global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
+template <int D, int NQ, int KSPLIT, int STAGES, int BLOCKS_PER_CU>
+// (the second launch bound counts waves per SIMD: a block of 256 KSPLIT threads puts KSPLIT on each)
+__global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos,
     bf16* __restrict__ out, int Hq, int Hkv, float scale, int window) {
-  constexpr int NT = 256 * KSPLIT;
+  constexpr int NT = 256 * KSPLIT, NW = NT / WAVE;
   constexpr int KK = D / 32, DB = D / 16;
   constexpr int ROWS = 64 * NQ;     // query rows per block
   constexpr int WROWS = 16 * NQ;    // per row group
   constexpr int WK = TK / KSPLIT;   // keys of a tile per wave
   constexpr int TB = WK / 16;       // 16-key blocks per wave and tile
-  constexpr int KS = D + 8;         // LDS row stride of the K tile (bf16)
-  constexpr int VS = TK + 8;        // LDS row stride of the V^T tile
+  constexpr int KROW = D * 2;       // bytes of a K row in LDS (no padding: the chunks are permuted instead)
+  constexpr int KCH = D / 8;        // its 16-byte chunks: 8 or 16
+  constexpr int KRPI = 1024 / KROW; // K rows one load instruction of a wave fills
+  constexpr int KI = TK / KRPI / NW;  // K load instructions per wave and tile
+  constexpr int VROW = TK * 2;      // bytes of a V^T row (one head element, 64 keys)
+  constexpr int VI = D / 8 / NW;    // V^T load instructions per wave and tile (8 rows each)
+  constexpr int K_BYTES = TK * KROW, STAGE_BYTES = K_BYTES + D * VROW;
+  static_assert(KI >= 1 && VI >= 1 && KI * KRPI * NW == TK && VI * 8 * NW == D, "head size and block size");
   // After the last tile the same memory carries the second key group's results to the first.
-  constexpr int TILE_BYTES = (TK * KS + D * VS) * 2;
-  constexpr int MERGE_BYTES = KSPLIT > 1 ? 4 * NQ * (16 * (D + 1) + 32) * 4 : 0;
-  __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES];
-  bf16* ks = reinterpret_cast<bf16*>(smem);
-  bf16* vs = ks + TK * KS;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // prefill_lds_bytes<D, NQ, KSPLIT, STAGES>()
 
   const int G = Hq / Hkv;
   const int kvh = blockIdx.x % Hkv, tile = blockIdx.x / Hkv;
@@ -143,28 +130,72 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
     for (int i = 0; i < DB; ++i) o[b][i] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // Global -> registers -> LDS with PD tiles in flight: a tile's loads are issued PD iterations before
-  // it is needed, since one iteration of products is much shorter than a trip to memory. The register
-  // sets rotate; the loop is unrolled PD-fold so that each set has a fixed name.
-  constexpr int PD = (KSPLIT == 1 && D == 128) ? 1 : 3;  // the widest variant has no registers to spare
-  u32x4 kreg[PD][TK * (D / 8) / NT], vreg[PD][TK * (D / 8) / NT];
+  // Chunk c of K row R lies in slot c ^ kswz(R) of the row, chunk c of V^T row d in slot c ^ ((d >> 1) & 7).
+  auto kswz = [](int R) { return KCH == 16 ? (R & 15) : ((R >> 1) & 7); };
+  // One tile's loads: wave-instruction q fills 1 KB of the stage in lane order. What does not depend on
+  // the tile is worked out once: the offset of the lane's chunk within its page, and which of the
+  // tile's four pages it comes from. Tiles past the last key are clamped to the last tile (what is
+  // fetched for them is never used); table entries without a page (past the last key, or given back
+  // behind a window) read page 0 instead: their keys are masked.
+  const size_t page_elems = (size_t)Hkv * PAGE * D;  // one page of K, and of V^T
+  int k_page[KI], v_page[VI];
+  unsigned k_off[KI], v_off[VI];
+#pragma unroll
+  for (int j = 0; j < KI; ++j) {
+    const int R = (wave * KI + j) * KRPI + lane / KCH, c = (lane % KCH) ^ kswz(R);
+    k_page[j] = __builtin_amdgcn_readfirstlane(R / PAGE);  // the rows of one instruction lie in one page
+    k_off[j] = (unsigned)((kvh * PAGE + R % PAGE) * D + c * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < VI; ++j) {
+    const int d = (wave * VI + j) * 8 + lane / 8, c = (lane % 8) ^ ((d >> 1) & 7);  // chunk c: keys 8 c .. 8 c + 7 of the tile
+    v_page[j] = c / 2;
+    v_off[j] = (unsigned)((kvh * D + d) * PAGE + (c % 2) * 8);
+  }
+  auto issue = [&](i32x4 pages, int stage_index) __attribute__((always_inline)) {
+    unsigned char* stage = smem + stage_index * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < KI; ++j) {
+      const bf16* src = kc + (size_t)max(pick(pages, k_page[j]), 0) * page_elems + k_off[j];
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                       (void __attribute__((address_space(3)))*)(stage + (wave * KI + j) * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < VI; ++j) {
+      const bf16* src = vc + (size_t)max(pick(pages, v_page[j]), 0) * page_elems + v_off[j];
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                       (void __attribute__((address_space(3)))*)(stage + K_BYTES + (wave * VI + j) * 1024), 16,
+                                       0, 0);
+    }
+  };
+
   const float scale2 = scale * 1.44269504088896340736f;  // scores in units of log2: exp2 is one instruction
   const int t_first = (kv_lo / TK) * TK;
+  const int n_tiles = (last_pos - t_first) / TK + 1;
+  // Issue order: page ids of tile m + 1, then the loads of tile m. At the top of iteration n the loads
+  // of tiles n + 1 .. n + STAGES - 2 may still be in flight, those of tile n must have landed.
+  i32x4 pages_next = tile_pages(table, t_first, last_pos);
 #pragma unroll
-  for (int st = 0; st < PD; ++st)
-    fetch_tile<D, NT>(kreg[st], vreg[st], kc, vc, tile_pages(table, t_first + st * TK, last_pos), t_first + st * TK, last_pos,
-                      Hkv, kvh, tid);
-  i32x4 pages_next = tile_pages(table, t_first + PD * TK, last_pos);
-  for (int tbase = t_first; tbase <= last_pos; tbase += PD * TK) {
-#pragma unroll
-  for (int st = 0; st < PD; ++st) {
-    const int t0 = tbase + st * TK;
-    if (t0 > last_pos) break;
-    __syncthreads();  // the previous tile has been consumed
-    stash_tile<D, NT>(kreg[st], vreg[st], ks, vs, tid);
-    __syncthreads();
-    fetch_tile<D, NT>(kreg[st], vreg[st], kc, vc, pages_next, t0 + PD * TK, last_pos, Hkv, kvh, tid);
-    pages_next = tile_pages(table, t0 + (PD + 1) * TK, last_pos);
+  for (int st = 0; st < STAGES - 1; ++st) {
+    const i32x4 pages = pages_next;
+    pages_next = tile_pages(table, t_first + (st + 1) * TK, last_pos);
+    issue(pages, st);
+  }
+  // This lane's key rows of a 32-key pair: product h (0 or 1) takes keys 4 h + {0-3, 8-11} of each of
+  // the pair's two pages, rows 0-7 from the first page and 8-15 from the second.
+  const int krow = (r < 8 ? 0 : 16) + (r % 4) + 8 * ((r / 4) % 2);
+  const int vsw = (r >> 1) & 7;
+  for (int n = 0; n < n_tiles; ++n) {
+    const int t0 = t_first + n * TK;
+    wait_loads<(STAGES - 2) * (KI + VI)>();
+    __syncthreads();  // tile n has landed for every wave, and every wave is done with tile n - 1
+    {
+      const i32x4 pages = pages_next;
+      pages_next = tile_pages(table, t0 + STAGES * TK, last_pos);
+      issue(pages, (n + STAGES - 1) % STAGES);
+    }
+    const unsigned char* ks = smem + (n % STAGES) * STAGE_BYTES;
+    const unsigned char* vs = ks + K_BYTES;
     const int w0 = t0 + kg * WK;  // this wave's keys of the tile: w0 .. w0 + WK - 1
     if (!grp_has_rows || w0 > grp_last_pos) continue;
     if (window > 0 && w0 + WK - 1 < grp_first_pos - window + 1) continue;
@@ -182,7 +213,10 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk)
-          kf[tb][kk] = *reinterpret_cast<const bf16x8*>(&ks[(kg * WK + tb * 16 + r) * KS + kk * 32 + g * 8]);
+        {
+          const int R = kg * WK + (tb / 2) * 32 + krow + 4 * (tb % 2);
+          kf[tb][kk] = *reinterpret_cast<const bf16x8*>(ks + R * KROW + (((kk * 4 + g) ^ kswz(R)) * 16));
+        }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk)  // consecutive products go to different accumulators
@@ -192,27 +226,35 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
           for (int b = 0; b < NQ; ++b) s[b][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tb][kk], qf[b][kk], s[b][tb], 0, 0, 0);
     }
     bf16x8 pf[NQ][TB / 2];
-    // Masks only where the keys cross the diagonal or the window's edge for some row of the group.
-    const bool masked = w0 + WK - 1 > grp_first_pos || (window > 0 && w0 <= grp_last_pos - window);
+    // Masks only where the keys cross the diagonal or the window's edge for some row of the group
+    // (the same answer for the whole wave: one branch around all of it).
+    const bool masked = __builtin_amdgcn_readfirstlane(
+        (int)(w0 + WK - 1 > grp_first_pos || (window > 0 && w0 <= grp_last_pos - window)));
+    if (masked) {
+#pragma unroll
+      for (int b = 0; b < NQ; ++b)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            // Scores of row r of block b: keys w0 + (tb / 2) * 32 + 8 g + 4 (tb % 2) + i.
+            const int t = w0 + (tb / 2) * 32 + 8 * g + 4 * (tb % 2) + i;
+            const bool seen = !row_ok[b] | ((t <= row_pos[b]) & ((window == 0) | (t > row_pos[b] - window)));
+            s[b][tb][i] = seen ? s[b][tb][i] : -INFINITY;
+          }
+    }
 #pragma unroll
     for (int b = 0; b < NQ; ++b) {
-      // Scores of row r of block b: tokens w0 + tb * 16 + 4 g + i.
       float m_new = m_run[b];
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = s[b][tb][i] * scale2;
-          if (masked) {
-            const int t = w0 + tb * 16 + 4 * g + i;
-            const bool seen = !row_ok[b] || (t <= row_pos[b] && (window == 0 || t > row_pos[b] - window));
-            v = seen ? v : -INFINITY;
-          }
+          const float v = s[b][tb][i] * scale2;  // -inf stays -inf (the scale is positive)
           s[b][tb][i] = v;
           m_new = fmaxf(m_new, v);
         }
-      m_new = fmaxf(m_new, __shfl_xor(m_new, 16, WAVE));
-      m_new = fmaxf(m_new, __shfl_xor(m_new, 32, WAVE));
+      m_new = rows4_max(m_new);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
       float psum = 0.f;
 #pragma unroll
@@ -223,52 +265,40 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
           psum += p;
           pf[b][tb / 2][(tb % 2) * 4 + i] = static_cast<bf16>(p);
         }
-      psum += __shfl_xor(psum, 16, WAVE);
-      psum += __shfl_xor(psum, 32, WAVE);
+      psum = rows4_sum(psum);
       const float corr = __builtin_amdgcn_exp2f(m_run[b] - m_safe);
       l_run[b] = l_run[b] * corr + psum;
       m_run[b] = m_new;
-      float cq[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) cq[i] = __shfl(corr, 4 * g + i, WAVE);
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[b][db][i] *= cq[i];
+        for (int i = 0; i < 4; ++i) o[b][db][i] *= corr;  // the lane's output values are all of its own row
     }
     {
-      // The same for the V^T fragments of the second product.
-      bf16x4 va[TB / 2][DB], vb[TB / 2][DB];
+      // The same for the V^T fragments of the second product: keys 8 g .. 8 g + 7 of the pair.
+      bf16x8 vf[TB / 2][DB];
 #pragma unroll
       for (int pr = 0; pr < TB / 2; ++pr)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const bf16* vp = &vs[(db * 16 + r) * VS + kg * WK + pr * 32 + 4 * g];
-          va[pr][db] = *reinterpret_cast<const bf16x4*>(vp);
-          vb[pr][db] = *reinterpret_cast<const bf16x4*>(vp + 16);
+          const int c = (kg * WK + pr * 32) / 8 + g;
+          vf[pr][db] = *reinterpret_cast<const bf16x8*>(vs + (db * 16 + r) * VROW + ((c ^ vsw) * 16));
         }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int pr = 0; pr < TB / 2; ++pr)
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          bf16x8 vf;
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            vf[i] = va[pr][db][i];
-            vf[4 + i] = vb[pr][db][i];
-          }
-#pragma unroll
-          for (int b = 0; b < NQ; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[b][pr], vf, o[b][db], 0, 0, 0);
-        }
+          for (int b = 0; b < NQ; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[pr][db], pf[b][pr], o[b][db], 0, 0, 0);
     }
   }
-  }
+  wait_loads<0>();  // the tiles fetched ahead past the end must not land in memory that is used otherwise
 
   if (KSPLIT > 1) {
     // The second key group hands its running maximum, sum and output to the first through LDS.
     // Layout per (row group, block): 16 rows x (D + 1) floats of output, then 16 maxima, then 16 sums.
-    __syncthreads();  // the last tile has been consumed
+    __syncthreads();  // the last tile has been consumed, and nothing is in flight any more
     float* mg = reinterpret_cast<float*>(smem);
     constexpr int PER = 16 * (D + 1) + 32;
 #pragma unroll
@@ -278,7 +308,7 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) base[(4 * g + i) * (D + 1) + db * 16 + r] = o[b][db][i];
+          for (int i = 0; i < 4; ++i) base[r * (D + 1) + db * 16 + 4 * g + i] = o[b][db][i];
         if (g == 0) {
           base[16 * (D + 1) + r] = m_run[b];
           base[16 * (D + 1) + 16 + r] = l_run[b];
@@ -297,31 +327,59 @@ __global__ __launch_bounds__(256 * KSPLIT, 2 / KSPLIT) void attn_prefill_kernel(
       l_run[b] = l_run[b] * f1 + l2 * f2;
       m_run[b] = m;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float a1 = __shfl(f1, 4 * g + i, WAVE), a2 = __shfl(f2, 4 * g + i, WAVE);
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int db = 0; db < DB; ++db) o[b][db][i] = o[b][db][i] * a1 + base[(4 * g + i) * (D + 1) + db * 16 + r] * a2;
-      }
+        for (int i = 0; i < 4; ++i) o[b][db][i] = o[b][db][i] * f1 + base[r * (D + 1) + db * 16 + 4 * g + i] * f2;
     }
   }
 
-  // o[b][db][i] = O[row 4 g + i of block b][d = db * 16 + r]
+  // o[b][db][i] = O[row r of block b][d = db * 16 + 4 g + i]
 #pragma unroll
   for (int b = 0; b < NQ; ++b) {
-    const float inv = 1.f / l_run[b];  // of row r; the rows written below are 4 g + i
+    const float inv = 1.f / l_run[b];
+    const int row = rg * WROWS + b * 16 + r;
+    const int tok = row / G;
+    if (tok < count && row < (ROWS / G) * G) {
+      bf16* dst = out + ((size_t)(first + tok) * Hq + kvh * G + row % G) * D + 4 * g;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float inv_i = __shfl(inv, 4 * g + i, WAVE);
-      const int row = rg * WROWS + b * 16 + 4 * g + i;
-      const int tok = row / G;
-      if (tok < count && row < (ROWS / G) * G) {
-        bf16* dst = out + ((size_t)(first + tok) * Hq + kvh * G + row % G) * D;
+      for (int db = 0; db < DB; ++db) {
+        bf16x4 v;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) dst[db * 16 + r] = static_cast<bf16>(o[b][db][i] * inv_i);
+        for (int i = 0; i < 4; ++i) v[i] = static_cast<bf16>(o[b][db][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + db * 16) = v;
       }
     }
   }
 }
+
+template <int D, int NQ, int KSPLIT, int STAGES>
+constexpr int prefill_lds_bytes() {
+  constexpr int tiles = STAGES * (TK * D * 2 + D * TK * 2);
+  constexpr int merge = KSPLIT > 1 ? 4 * NQ * (16 * (D + 1) + 32) * 4 : 0;
+  return tiles > merge ? tiles : merge;
+}
+
+template <int D, int NQ, int KSPLIT, int STAGES, int BLOCKS_PER_CU>
+static int launch_prefill(unsigned grid, const bf16* q, int q_stride, const bf16* kc, const bf16* vc, const int* block_table,
+                          int table_width, const int* tile_first, const int* tile_count, const int* token_row,
+                          const int* pos, bf16* out, int Hq, int Hkv, float scale, int window, hipStream_t st) {
+  constexpr int lds = prefill_lds_bytes<D, NQ, KSPLIT, STAGES>();
+  static_assert(lds * BLOCKS_PER_CU <= 160 * 1024, "LDS of the blocks that share a CU");
+  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)attn_prefill_kernel<D, NQ, KSPLIT, STAGES, BLOCKS_PER_CU>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  attn_prefill_kernel<D, NQ, KSPLIT, STAGES, BLOCKS_PER_CU><<<grid, 256 * KSPLIT, lds, st>>>(q, q_stride, kc, vc, block_table, table_width,
+                                                                              tile_first, tile_count, token_row, pos, out,
+                                                                              Hq, Hkv, scale, window);
+  return launch_status();
+}
+#define PREFILL_ARGS                                                                                                    \
+  (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, \
+      pos, (bf16*)out, Hq, Hkv, scale, window, st
 
 // Tokens per tile for a group of G query heads per KV head and `rows` query rows per block.
 extern "C" int ms_attention_prefill_tile_tokens(int G, int rows) { return G >= 1 && G <= rows ? rows / G : 0; }
@@ -340,15 +398,10 @@ extern "C" int ms_attention_prefill_bf16(const void* q, int q_stride, const void
       (rows_per_tile != 64 && rows_per_tile != 128))
     return MS_BAD_ARG;
   const unsigned grid = (unsigned)tiles * Hkv;
-#define LAUNCH(DD, NN, KS_)                                                                                       \
-  attn_prefill_kernel<DD, NN, KS_><<<grid, 256 * KS_, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc,         \
-                                                               (const bf16*)vc, block_table, table_width,         \
-                                                               tile_first, tile_count, token_row, pos,            \
-                                                               (bf16*)out, Hq, Hkv, scale, window)
-  if (D == 128 && rows_per_tile == 128) LAUNCH(128, 2, 1);
-  else if (D == 128) LAUNCH(128, 1, 2);
-  else if (rows_per_tile == 128) LAUNCH(64, 2, 1);
-  else LAUNCH(64, 1, 2);
-#undef LAUNCH
-  return launch_status();
+  // Two stages were as fast as four in every shape tried (the loop is bound by its instructions, not
+  // by the loads), and leave room for two blocks per CU.
+  if (D == 128 && rows_per_tile == 128) return launch_prefill<128, 2, 1, 2, 2>(grid, PREFILL_ARGS);
+  if (D == 128) return launch_prefill<128, 1, 2, 2, 2>(grid, PREFILL_ARGS);
+  if (rows_per_tile == 128) return launch_prefill<64, 2, 1, 2, 2>(grid, PREFILL_ARGS);
+  return launch_prefill<64, 1, 2, 2, 2>(grid, PREFILL_ARGS);
 }

@@ -34,6 +34,22 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Sum over a block of NT threads (NT a multiple of 64, at most 1024). `red` holds NT / 64 floats.
 // Every thread receives the total; the order of additions is fixed by NT alone.
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one element of each 16-lane row), the
+// same bits in all four: v_permlane16_swap and v_permlane32_swap hand a lane its partner's value
+// without a trip through LDS. The sum is (row 0 + row 1) + (row 2 + row 3) for every lane.
+__device__ __forceinline__ float rows4_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows4_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;

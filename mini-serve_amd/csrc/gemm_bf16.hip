@@ -263,19 +263,26 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
     __syncthreads();  // slab k has landed for every wave, and every wave is done with slab k - 1
     if (k + STAGES - 1 < slabs) issue(k + STAGES - 1);
     const unsigned char* stage = lds + (k % STAGES) * STAGE_BYTES;
+    // All fragments of the slab are asked for before the first product (the scheduler is told not to
+    // move them back down): the reads return in order, so each product waits only for its own
+    // operands while the later reads are still on their way.
+    constexpr int STEPS = CPR / 4;
+    bf16x8 wf[STEPS][FN], xf[STEPS][FM];
 #pragma unroll
-    for (int kk = 0; kk < CPR; kk += 4) {  // chunk columns kk + g
-      const int slot = ((kk + g) ^ sw) * 16;
-      bf16x8 wf[FN], xf[FM];
+    for (int t = 0; t < STEPS; ++t) {
+      const int slot = ((t * 4 + g) ^ sw) * 16;  // chunk column 4 t + g
 #pragma unroll
-      for (int i = 0; i < FN; ++i) wf[i] = *reinterpret_cast<const bf16x8*>(stage + w_off + i * 16 * ROW_BYTES + slot);
+      for (int i = 0; i < FN; ++i) wf[t][i] = *reinterpret_cast<const bf16x8*>(stage + w_off + i * 16 * ROW_BYTES + slot);
 #pragma unroll
-      for (int j = 0; j < FM; ++j) xf[j] = *reinterpret_cast<const bf16x8*>(stage + x_off + j * 16 * ROW_BYTES + slot);
+      for (int j = 0; j < FM; ++j) xf[t][j] = *reinterpret_cast<const bf16x8*>(stage + x_off + j * 16 * ROW_BYTES + slot);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t)
 #pragma unroll
       for (int i = 0; i < FN; ++i)
 #pragma unroll
-        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[j], acc[i][j], 0, 0, 0);
-    }
+        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
   }
 
   const bool vec_store = (ldc % 4 == 0);

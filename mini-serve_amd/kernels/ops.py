@@ -370,7 +370,7 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
     return page
 
 
-PREFILL_BIG_BLOCKS = 1024  # from this many 128-row blocks on, the prefill attention runs 128-row blocks
+PREFILL_BIG_BLOCKS = 640  # from this many 128-row blocks on, the prefill attention runs 128-row blocks
 DECODE_TARGET_BLOCKS = 512  # workgroups the split decode kernel aims for
 DECODE_MIN_CHUNKS = 4  # 32-token chunks a split should at least hold
 
@@ -399,6 +399,8 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
         raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} KV heads")
     if qkv.shape[1] < num_heads * head_dim:
         raise ValueError("qkv is narrower than the query heads")
+    if not scale > 0:
+        raise ValueError(f"the attention scale must be positive, not {scale}")  # the kernels scale masked scores too
     _dev(block_table, "block_table", I32, 2)
     _dev(batch.token_row, "token_row", I32, 1)
     _dev(batch.positions, "positions", I32, 1)
