@@ -67,6 +67,9 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     }
   }
 
+  // Scores are kept in units of log2 (exp2 is one instruction); maxima, also those handed to the
+  // reduction kernel, are in the same units.
+  const float scale2 = scale * 1.44269504088896340736f;
   float m_run = -INFINITY, l_run = 0.f;  // of query r (replicated over the four lane groups)
   floatx4 o[DB];
 #pragma unroll
@@ -117,8 +120,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int ta = tl + i, tb = ta + 4;
-      sc[i] = (ta >= lo && ta < kv_len) ? s0[i] * scale : -INFINITY;
-      sc[4 + i] = (tb >= lo && tb < kv_len) ? s1[i] * scale : -INFINITY;
+      sc[i] = (ta >= lo && ta < kv_len) ? s0[i] * scale2 : -INFINITY;
+      sc[4 + i] = (tb >= lo && tb < kv_len) ? s1[i] * scale2 : -INFINITY;
       m_new = fmaxf(m_new, fmaxf(sc[i], sc[4 + i]));
     }
     m_new = rows4_max(m_new);
@@ -128,12 +131,12 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     bf16x8 pf;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float p = expf(sc[i] - m_new);
+      const float p = __builtin_amdgcn_exp2f(sc[i] - m_new);
       psum += p;
       pf[i] = static_cast<bf16>(p);
     }
     psum = rows4_sum(psum);
-    const float corr = expf(m_run - m_new);
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
     l_run = l_run * corr + psum;
     m_run = m_new;
     // O^T[d, query]: a lane's output values are all of its own query r.
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     if (M > -INFINITY) {
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        const float f = expf(sm[w][qh] - M);  // 0 for a wave that saw nothing
+        const float f = __builtin_amdgcn_exp2f(sm[w][qh] - M);  // 0 for a wave that saw nothing
         L += sl[w][qh] * f;
         O += so[w][qh][d] * f;
       }
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __re
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-      const float f = q[u].x == -INFINITY ? 0.f : expf(q[u].x - M);  // an empty or absent split adds nothing
+      const float f = q[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(q[u].x - M);  // an empty or absent split adds nothing
       L += q[u].y * f;
       O += o[u] * f;
     }
