@@ -93,9 +93,10 @@ def test_rmsnorm_eps_enters(ops):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-def test_silu_mul(ops, dtype):
-    gu = rand((5, 2 * 224), dtype, 5, 2.0)
-    g, u = gu[:, :224].double(), gu[:, 224:].double()
+@pytest.mark.parametrize("inter", [224, 100, 3072])  # a multiple of 8 moves vectors, others single elements
+def test_silu_mul(ops, dtype, inter):
+    gu = rand((5, 2 * inter), dtype, 5, 2.0)
+    g, u = gu[:, :inter].double(), gu[:, inter:].double()
     want = g / (1 + torch.exp(-g)) * u
     close(ops.act_mul(gu), want, 1e-6 if dtype == F32 else 5e-3, "silu_mul")
     z = torch.zeros((1, 8), dtype=dtype, device=DEV)
