@@ -1,8 +1,9 @@
 """A toy architecture, defined entirely in this test, is registered, built and stepped without a
-change to the framework's files: a mixer with fixed-size per-request state of its own, a run order
-that names one layer's weights twice and lets an entry read another entry's cache, and a second
-position-free attention layer. Whole prompts, portions, single tokens and captured decode graphs
-must all agree with a plain implementation of the same toy, also defined here."""
+change to the framework's files: a mixer with fixed-size per-request state of its own, a feed-forward
+that routes each token to one of three experts, a position encoding of its own inside the stock
+attention mixer, and a run order that names one layer's weights twice and lets an entry read another
+entry's cache. Whole prompts, portions, single tokens and captured decode graphs must all agree with
+a plain implementation of the same toy, also defined here."""
 
 from __future__ import annotations
 
@@ -15,12 +16,14 @@ from plain import qwen3_plain as P
 pytestmark = pytest.mark.gpu
 
 H, HEADS, KVH, D, INTER, VOCAB, DECAY = 64, 4, 2, 16, 96, 97, 0.75
+EXPERTS, EXPERT_WIDTH, ROUTER_SCALE = 3, 32, 60.0  # the scale keeps the winner clear of bfloat16 rounding
+ROT_DIM, POS_STEP = 8, 0.5  # the toy position encoding turns pair j of the first 8 elements by (POS_STEP * position) / (j + 1)
 
 
 @pytest.fixture(scope="module")
 def toy():
     from miniserve_amd.config import LayerSpec, ModelSpec, PartSpec, RunEntry, register_architecture, unregister_architecture
-    from miniserve_amd.parts import Mixer, StateNeed, TensorSpec, register, unregister
+    from miniserve_amd.parts import FeedForward, Mixer, PositionEncoding, Rotation, StateNeed, TensorSpec, register, unregister
 
     @register("mixer", "toy_decay")
     class DecayMixer(Mixer):
@@ -60,6 +63,56 @@ def toy():
                     t += n
             return self.rt.ops.linear(out.to(x.dtype).contiguous(), self.weight, accumulate_into=residual, defer=True)
 
+    @register("feed_forward", "toy_routed")
+    class RoutedFeedForward(FeedForward):
+        """Each token goes to the expert with the largest router logit (float32) and gets that expert's
+        ``W2 relu(W1 x)`` times the router's softmax weight of it. All experts are run and the others'
+        hidden units zeroed: no host decision, so a decode step can be captured."""
+
+        def __init__(self, spec, rt):
+            super().__init__(spec, rt)
+            self.width, self.experts, self.inner = int(spec["width"]), int(spec["experts"]), int(spec["inner"])
+            self.router_scale = float(spec["router_scale"])
+
+        @classmethod
+        def tensors(cls, spec):
+            w, e, f = int(spec["width"]), int(spec["experts"]), int(spec["inner"])
+            return {"moe.router.weight": TensorSpec((e, w)), "moe.w1.weight": TensorSpec((e * f, w)),
+                    "moe.w2.weight": TensorSpec((w, e * f))}
+
+        def bind(self, tensors):
+            self.router, self.w1, self.w2 = (tensors["moe." + n + ".weight"] for n in ("router", "w1", "w2"))
+            self.expert_ids = torch.arange(self.experts, device=self.router.device)
+
+        def forward(self, x, residual):
+            ops = self.rt.ops
+            logits = (x.float() @ self.router.float().T) * self.router_scale
+            prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            hidden = torch.relu(ops.linear(x, self.w1, out_dtype=self.rt.dtype)).view(-1, self.experts, self.inner)
+            chosen = (choice[:, None] == self.expert_ids[None, :]).to(hidden.dtype)[:, :, None]
+            y = ops.linear((hidden * chosen).view(-1, self.experts * self.inner).contiguous(), self.w2, out_dtype=torch.float32)
+            residual += prob[:, None] * y
+            return None
+
+        def parameters_bytes(self):
+            return sum(t.numel() * t.element_size() for t in (self.router, self.w1, self.w2))
+
+    @register("position", "toy_slow_rotation")
+    class SlowRotation(PositionEncoding):
+        """Pair j of the first ``dim`` elements of a head is turned by ``step * position / (j + 1)``."""
+
+        def __init__(self, spec, rt):
+            super().__init__(spec, rt)
+            self.dim, self.step = int(spec["dim"]), float(spec["step"])
+
+        def rotation(self, batch):
+            key = ("toy_slow_rotation", self.dim, self.step)
+            if key not in batch.memo:
+                j = torch.arange(1, self.dim // 2 + 1, device=batch.positions.device, dtype=torch.float32)
+                ang = (batch.positions.float() * self.step)[:, None] / j[None, :]
+                batch.memo[key] = torch.cat((torch.cos(ang), torch.sin(ang)), dim=1).contiguous()
+            return Rotation(self.dim, batch.memo[key])
+
     @register_architecture("ToyForCausalLM")
     class ToyConfig:
         @classmethod
@@ -79,9 +132,11 @@ def toy():
             ffn = PartSpec("gated_mlp", {"prefix": "mlp.", "hidden_size": H, "intermediate_size": INTER, "activation": "silu"})
             attn = PartSpec("gqa_attention", {
                 "prefix": "attn.", "hidden_size": H, "num_heads": HEADS, "num_kv_heads": KVH, "head_dim": D,
-                "scale": 0.3, "qk_norm_eps": None, "window": 0, "position": PartSpec("rotary", {"dim": 8, "theta": 100.0})})
+                "scale": 0.3, "qk_norm_eps": None, "window": 0,
+                "position": PartSpec("toy_slow_rotation", {"dim": ROT_DIM, "step": POS_STEP})})
+            routed = PartSpec("toy_routed", {"width": H, "experts": EXPERTS, "inner": EXPERT_WIDTH, "router_scale": ROUTER_SCALE})
             layers = (
-                LayerSpec("l0.", block(), PartSpec("toy_decay", {"width": H, "decay": DECAY}), ffn),
+                LayerSpec("l0.", block(), PartSpec("toy_decay", {"width": H, "decay": DECAY}), routed),
                 LayerSpec("l1.", block(), attn, ffn),
             )
             order = (RunEntry(0, 0), RunEntry(1, 1), RunEntry(1, 2), RunEntry(1, 1, writes_cache=False))
@@ -94,11 +149,17 @@ def toy():
     yield ToyConfig
     unregister_architecture("ToyForCausalLM")
     unregister("mixer", "toy_decay")
+    unregister("feed_forward", "toy_routed")
+    unregister("position", "toy_slow_rotation")
+
+
+margins: list[float] = []  # smallest gap between the two best router logits of each sequence the plain toy ran
 
 
 def plain_toy(w, ids):
-    """The toy in float64: layer 0 (decay mixer), then layer 1's weights three times: with a cache of
-    its own, with another cache of its own, and reading the keys and values of the first of these."""
+    """The toy in float64: layer 0 (decay mixer, routed feed-forward), then layer 1's weights three
+    times: with a cache of its own, with another cache of its own, and reading the keys and values of
+    the first of these."""
     w = {k: v.double().cpu().numpy() for k, v in w.items()}
     T = len(ids)
     h = w["emb.weight"][np.asarray(ids)]
@@ -112,12 +173,24 @@ def plain_toy(w, ids):
     for t in range(T):
         s = DECAY * s + x[t]
         outs.append(s)
-    h = mlp(h + np.stack(outs) @ w["l0.toy.weight"].T, "l0.")
+    h = h + np.stack(outs) @ w["l0.toy.weight"].T
+    # routed feed-forward: the expert with the largest router logit, weighted by its softmax weight
+    y = P.rms_norm(h, w["l0.n2.weight"], 1e-5)
+    logits = (y @ w["l0.moe.router.weight"].T) * ROUTER_SCALE
+    prob = np.exp(logits - logits.max(-1, keepdims=True))
+    prob /= prob.sum(-1, keepdims=True)
+    choice = logits.argmax(-1)
+    ranked = np.sort(logits, axis=-1)
+    margins.append(float((ranked[:, -1] - ranked[:, -2]).min()))
+    w1 = w["l0.moe.w1.weight"].reshape(EXPERTS, EXPERT_WIDTH, H)
+    w2 = w["l0.moe.w2.weight"].reshape(H, EXPERTS, EXPERT_WIDTH)
+    out = np.stack([prob[t, e] * (w2[:, e, :] @ np.maximum(w1[e] @ y[t], 0.0)) for t, e in enumerate(choice)])
+    h = h + out
 
-    ang = P.rotary_angles(np.arange(T), 8, 100.0)
+    ang = ((np.arange(T) * POS_STEP)[:, None] / np.arange(1, ROT_DIM // 2 + 1)[None, :]).astype(np.float32)
 
-    def rot(v):  # partial rotation: the first 8 elements of each head
-        return np.concatenate((P.apply_rotary(v[..., :8], ang), v[..., 8:]), axis=-1)
+    def rot(v):  # partial rotation: the first ROT_DIM elements of each head
+        return np.concatenate((P.apply_rotary(v[..., :ROT_DIM], ang), v[..., ROT_DIM:]), axis=-1)
 
     def qkv(h):
         x = P.rms_norm(h, w["l1.n1.weight"], 1e-5)
@@ -162,7 +235,10 @@ def test_toy_architecture_runs_through_the_engine(toy, dtype):
     assert [g.slots for g in runner.layout.groups] == [(1, 2)] and [s.slot for s in runner.layout.states] == [0]
     rng = np.random.default_rng(3)
     seqs = [rng.integers(0, VOCAB, n).tolist() for n in (37, 50, 9)]
+    margins.clear()
     want = [plain_toy(weights, ids) for ids in seqs]
+    # The comparison below means something only where rounding cannot change an expert choice.
+    assert min(margins) > (0.5 if dtype == "bfloat16" else 1e-3), f"router margins {margins}: pick another seed"
 
     def feed(rc, ids, at, n, wanted):
         return StepRow(rc, ids[at : at + n], wanted)
