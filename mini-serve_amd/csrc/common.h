@@ -32,8 +32,6 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// Sum over a block of NT threads (NT a multiple of 64, at most 1024). `red` holds NT / 64 floats.
-// Every thread receives the total; the order of additions is fixed by NT alone.
 // Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one element of each 16-lane row), the
 // same bits in all four: v_permlane16_swap and v_permlane32_swap hand a lane its partner's value
 // without a trip through LDS. The sum is (row 0 + row 1) + (row 2 + row 3) for every lane.
@@ -50,6 +48,8 @@ __device__ __forceinline__ float rows4_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// Sum over a block of NT threads (NT a multiple of 64, at most 1024). `red` holds NT / 64 floats.
+// Every thread receives the total; the order of additions is fixed by NT alone.
 template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
