@@ -285,6 +285,28 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
         for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
   }
 
+  if (mode == 3) {
+    // Gated epilogue: W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and
+    // 2 p + 1 of a lane are gate and up of the same four outputs: out[m, n / 2 ...] = silu(gate) * up,
+    // bf16 [M, N / 2] with row stride ldc.
+    static_assert(FN % 2 == 0, "gate and up fragments come in pairs");
+#pragma unroll
+    for (int i = 0; i < FN; i += 2)
+#pragma unroll
+      for (int j = 0; j < FM; ++j) {
+        const int m = m0 + wm + j * 16 + r, col = (n0 + wn + i * 16) / 2 + g * 4;
+        if (m < M && col < N / 2) {
+          union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float gate = acc[i][j][e];
+            o.e[e] = static_cast<bf16>(gate / (1.f + expf(-gate)) * acc[i + 1][j][e]);
+          }
+          *reinterpret_cast<uint2*>((bf16*)Cbase + (size_t)m * ldc + col) = o.u;
+        }
+      }
+    return;
+  }
   const bool vec_store = (ldc % 4 == 0);
 #pragma unroll
   for (int i = 0; i < FN; ++i)
@@ -539,6 +561,95 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
     splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);
   }
   return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gated feed-forward input for few rows (M <= 16): out[m, i] = silu(x . gate_i) * (x . up_i), bf16
+// [M, inter], from W [2 inter, K] that holds alternating blocks of 16 gate rows and 16 up rows. One
+// block of 4 waves per 16 outputs: wave w takes K slabs w, w + 4, ... of the 32 weight rows (their
+// loads all in flight at once), the four partial results meet in LDS and wave 0 adds them in wave
+// order, applies the activation and stores. No partial sums leave the block and no second kernel
+// runs. K must be a multiple of 256 and rows 16-byte aligned.
+__global__ __launch_bounds__(256) void gemm_bf16_small_gated_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                                    bf16* __restrict__ out, int M, int inter, int K,
+                                                                    int ldx) {
+  __shared__ float red[4][2][WAVE][4];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int nb = blockIdx.x * 32;  // first weight row of the pair of blocks
+  floatx4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+  const bf16* wg = W + (size_t)(nb + r) * K + g * 16;
+  const bf16* wu = wg + (size_t)16 * K;
+  const bf16* xp = X + (size_t)min(r, M - 1) * ldx + g * 16;  // rows beyond M: read row M - 1, use zeros
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int k0 = wave * SMALL_SLAB; k0 < K; k0 += 4 * SMALL_SLAB) {
+    Chunk a[SMALL_SLAB / 64][2], b[SMALL_SLAB / 64][2], x[SMALL_SLAB / 64][2];
+#pragma unroll
+    for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+      a[u][0].u = *reinterpret_cast<const uint4*>(wg + k0 + u * 64);
+      a[u][1].u = *reinterpret_cast<const uint4*>(wg + k0 + u * 64 + 8);
+      b[u][0].u = *reinterpret_cast<const uint4*>(wu + k0 + u * 64);
+      b[u][1].u = *reinterpret_cast<const uint4*>(wu + k0 + u * 64 + 8);
+    }
+#pragma unroll
+    for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+      const uint4 lo = *reinterpret_cast<const uint4*>(xp + k0 + u * 64);
+      const uint4 hi = *reinterpret_cast<const uint4*>(xp + k0 + u * 64 + 8);
+      x[u][0].u = r < M ? lo : zero;
+      x[u][1].u = r < M ? hi : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < SMALL_SLAB / 64; ++u) {
+      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][0].v, x[u][0].v, acc_g, 0, 0, 0);
+      acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][0].v, x[u][0].v, acc_u, 0, 0, 0);
+      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][1].v, x[u][1].v, acc_g, 0, 0, 0);
+      acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][1].v, x[u][1].v, acc_u, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    red[wave][0][lane][e] = acc_g[e];
+    red[wave][1][lane][e] = acc_u[e];
+  }
+  __syncthreads();
+  if (wave != 0 || r >= M) return;
+  // This lane: outputs 16 blockIdx.x + 4 g + e of row m = r.
+  union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float gate = 0.f, up = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      gate += red[w][0][lane][e];
+      up += red[w][1][lane][e];
+    }
+    o.e[e] = static_cast<bf16>(gate / (1.f + expf(-gate)) * up);
+  }
+  *reinterpret_cast<uint2*>(out + (size_t)r * inter + blockIdx.x * 16 + g * 4) = o.u;
+}
+
+// out bf16 [M, inter] = silu(X gate^T) * (X up^T) for W [2 inter, K] with gate and up rows in
+// alternating blocks of 16. MS_UNSUPPORTED for shapes no fused kernel takes (the caller then runs the
+// product and the activation separately): K no multiple of 64 (of 256 for M <= 16) or unaligned rows,
+// 17 <= M <= 64 (those stream the weights with K split over blocks), more K than a block of the small
+// kernel should walk alone.
+extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M, int inter, int K, int ldx, hipStream_t st) {
+  if (M <= 0 || inter <= 0) return MS_OK;
+  if (K <= 0 || ldx < K) return MS_BAD_ARG;
+  if (inter % 16 || ldx % 8) return MS_UNSUPPORTED;
+  const bf16* x = (const bf16*)X;
+  const bf16* w = (const bf16*)W;
+  const int N = 2 * inter;
+  if (M <= 16) {
+    if (K % SMALL_SLAB || K / SMALL_SLAB > 8) return MS_UNSUPPORTED;
+    gemm_bf16_small_gated_kernel<<<inter / 16, 256, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    return launch_status();
+  }
+  if (M <= 64 || K % BK) return MS_UNSUPPORTED;
+  const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (big >= 256) return launch_dma<128, 128, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  if ((long)((M + 63) / 64) * ((N + 63) / 64) >= 256) return launch_dma<64, 64, BK, 2, 4>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  return MS_UNSUPPORTED;  // too few tiles without a split of K
 }
 
 // Splits of K for the tile kernel when the caller takes partial sums: as many as fill the chip with

@@ -23,8 +23,9 @@ _ERRORS = {1: "bad argument", 2: "unsupported size", 3: "kernel launch failed"}
 _SIGNATURES = {
     "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
     "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int, _c_ll, _c_void],
-    "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
-    "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
     "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
@@ -169,33 +170,73 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: 
     return out
 
 
-def act_mul(gu, activation: str = "silu", out_dtype=None) -> torch.Tensor:
-    """``act(gu[:, :I]) * gu[:, I:]`` for ``gu [T, 2 I]``, a tensor or a ``SplitSum`` (then ``out_dtype``
-    names the result's dtype)."""
+GATE_BLOCK = 16  # rows per run of gate / up rows in an interleaved gate-up weight
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``[2 I, K]`` with alternating runs of ``GATE_BLOCK`` gate rows and ``GATE_BLOCK`` up rows: the
+    order in which the matrix kernels hold gate and up of one output in one lane. ``I`` must be a
+    multiple of ``GATE_BLOCK``."""
+    i, k = gate.shape
+    if up.shape != gate.shape or i % GATE_BLOCK:
+        raise ValueError(f"gate {tuple(gate.shape)} and up {tuple(up.shape)} cannot be interleaved in runs of {GATE_BLOCK}")
+    both = torch.stack((gate.view(i // GATE_BLOCK, GATE_BLOCK, k), up.view(i // GATE_BLOCK, GATE_BLOCK, k)), dim=1)
+    return both.reshape(2 * i, k).contiguous()
+
+
+def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> torch.Tensor:
+    """``act(gate) * up`` for ``gu [T, 2 I]``, a tensor or a ``SplitSum`` (then ``out_dtype`` names the
+    result's dtype). ``block == 0``: the row holds the ``I`` gates, then the ``I`` ups; ``block > 0``:
+    alternating runs of ``block`` gates and ``block`` ups (see ``interleave_gate_up``)."""
     if activation != "silu":
         raise NotImplementedError(f"activation {activation!r}")
     if isinstance(gu, SplitSum):
         _dev(gu.parts, "gu", F32, 3)
         t, width = gu.shape
-        if width % 2 or out_dtype not in (F32, BF16):
-            raise ValueError("gate/up partial sums need an even width and an output dtype")
+        if width % 2 or out_dtype not in (F32, BF16) or (block and (width // 2) % block):
+            raise ValueError("gate/up partial sums need an even width (whole runs) and an output dtype")
         out = torch.empty((t, width // 2), dtype=out_dtype, device=gu.parts.device)
         for t0 in range(0, t, 32768):
             n = min(32768, t - t0)
             _check(library().ms_silu_mul_parts(gu.parts[:, t0:].data_ptr(), gu.splits, gu.stride, out[t0:].data_ptr(),
-                                               int(out_dtype == BF16), n, width // 2, _stream()), "silu_mul")
+                                               int(out_dtype == BF16), n, width // 2, int(block), _stream()), "silu_mul")
         return out
     _dev(gu, "gu", (F32, BF16), 2)
-    if gu.shape[1] % 2:
-        raise ValueError("gate/up buffer needs an even width")
+    if gu.shape[1] % 2 or (block and (gu.shape[1] // 2) % block):
+        raise ValueError("gate/up buffer needs an even width (whole runs)")
     inter = gu.shape[1] // 2
     out = torch.empty((gu.shape[0], inter), dtype=gu.dtype, device=gu.device)
     # grid.y carries the token index: split very long batches
     for t0 in range(0, gu.shape[0], 32768):
         n = min(32768, gu.shape[0] - t0)
-        _check(library().ms_silu_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, _stream()),
-               "silu_mul")
+        _check(library().ms_silu_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, int(block),
+                                     _stream()), "silu_mul")
     return out
+
+
+def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu", out_dtype=None, block: int = 0):
+    """``act(x gate^T) * (x up^T)`` for ``gate_up [2 I, K]`` laid out as ``act_mul`` describes. With
+    interleaved bfloat16 weights the activation runs in the matrix kernel's epilogue where a kernel
+    for the shape exists (few rows: no partial sums leave the kernel; many rows: the gate/up matrix is
+    never written); otherwise the product and the activation are two kernels."""
+    if activation != "silu":
+        raise NotImplementedError(f"activation {activation!r}")
+    _dev(x, "x", (F32, BF16), 2)
+    _dev(gate_up, "gate_up", (F32, BF16), 2)
+    m, k = x.shape
+    if gate_up.shape[1] != k or gate_up.shape[0] % 2:
+        raise ValueError(f"gated_linear: x is [{m}, {k}], gate_up is {tuple(gate_up.shape)}")
+    inter = gate_up.shape[0] // 2
+    if block == GATE_BLOCK and gate_up.dtype == BF16 and out_dtype == BF16 and m > 0:
+        xa = cast(x, BF16)
+        out = torch.empty((m, inter), dtype=BF16, device=x.device)
+        rc = library().ms_gemm_bf16_gated(xa.data_ptr(), gate_up.data_ptr(), out.data_ptr(), m, inter, k, k, _stream())
+        if rc == 0:
+            return out
+        if rc != 2:  # 2: no fused kernel for this shape
+            _check(rc, "gemm_bf16_gated")
+    gu = linear(x, gate_up, out_dtype=out_dtype, defer=True)
+    return act_mul(gu, activation, out_dtype=out_dtype, block=block)
 
 
 def cast(x: torch.Tensor, dtype) -> torch.Tensor:

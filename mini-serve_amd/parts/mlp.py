@@ -1,7 +1,9 @@
 """Gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases
-(miniserve/model/qwen3.py:128-131). Gate and up are one matrix product over row-concatenated
-weights ``[gate; up]`` (miniserve/model/fused.py:41,195); the activation product is evaluated in
-float32 and rounded once; the down projection adds into the residual stream in its epilogue."""
+(miniserve/model/qwen3.py:128-131). Gate and up are one matrix product over one weight that holds
+both (the reference concatenates them, miniserve/model/fused.py:41,195; here their rows alternate in
+runs of 16 where the width allows, so that a matrix kernel's lane holds gate and up of the same output
+and can finish the activation itself); the activation product is evaluated in float32 and rounded
+once; the down projection adds into the residual stream in its epilogue."""
 
 from __future__ import annotations
 
@@ -25,6 +27,7 @@ class GatedMLP(FeedForward):
         if self.activation not in ACTIVATIONS:
             raise NotImplementedError(f"activation {self.activation!r} is not supported, expected {ACTIVATIONS}")
         self.gate_up = self.down = None
+        self.block = 0  # rows per run of gate / up rows in gate_up (0: all gates, then all ups)
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -41,13 +44,14 @@ class GatedMLP(FeedForward):
         g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
         if g.dtype != u.dtype:
             raise ValueError(f"{p}gate/up projections are stored in different dtypes")
-        self.gate_up = torch.cat((g, u), dim=0).contiguous()
+        ops = self.rt.ops
+        self.block = ops.GATE_BLOCK if self.inter % ops.GATE_BLOCK == 0 else 0
+        self.gate_up = ops.interleave_gate_up(g, u) if self.block else torch.cat((g, u), dim=0).contiguous()
         self.down = tensors[p + "down_proj.weight"]
 
     def forward(self, x, residual):
         ops = self.rt.ops
-        gu = ops.linear(x, self.gate_up, out_dtype=self.rt.dtype, defer=True)
-        m = ops.act_mul(gu, self.activation, out_dtype=self.rt.dtype)
+        m = ops.gated_linear(x, self.gate_up, self.activation, out_dtype=self.rt.dtype, block=self.block)
         return ops.linear(m, self.down, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:

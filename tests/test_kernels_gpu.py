@@ -101,6 +101,34 @@ def test_silu_mul(ops, dtype, inter):
     close(ops.act_mul(gu), want, 1e-6 if dtype == F32 else 5e-3, "silu_mul")
     z = torch.zeros((1, 8), dtype=dtype, device=DEV)
     assert float(ops.act_mul(z).abs().max()) == 0.0
+    if inter % 16 == 0:  # the same values with gates and ups in alternating runs of 16
+        mixed = torch.stack((gu[:, :inter].reshape(5, inter // 16, 16), gu[:, inter:].reshape(5, inter // 16, 16)), dim=2)
+        close(ops.act_mul(mixed.reshape(5, 2 * inter).contiguous(), block=16), want, 1e-6 if dtype == F32 else 5e-3, "runs of 16")
+        parts = torch.stack([mixed.reshape(5, 2 * inter).float() * f for f in (0.5, 0.25, 0.25)])
+        close(ops.act_mul(ops.SplitSum(parts), out_dtype=dtype, block=16), want, 1e-6 if dtype == F32 else 5e-3, "partial sums")
+
+
+# (rows, width of x, outputs): few rows run one fused kernel whose waves split K and meet in LDS; many
+# rows the tile kernels with the activation in their epilogue; 17-64 rows, few tiles, a K that is no
+# multiple of 64, or float32 run the product and the activation as two kernels. All must agree.
+GATED = [(1, 1024, 3072), (8, 1024, 3072), (16, 512, 64), (5, 2048, 160), (13, 4096, 48), (40, 1024, 3072), (64, 256, 64),
+         (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096)]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("m,k,inter", GATED)
+def test_gated_linear(ops, dtype, m, k, inter):
+    x = rand((m, k), dtype, 70)
+    gate, up = rand((inter, k), dtype, 71, 0.05), rand((inter, k), dtype, 72, 0.05)
+    g, u = x.double() @ gate.double().T, x.double() @ up.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    w = ops.interleave_gate_up(gate, up)
+    assert w.shape == (2 * inter, k) and torch.equal(w[:16], gate[:16]) and torch.equal(w[16:32], up[:16])
+    got = ops.gated_linear(x, w, out_dtype=dtype, block=ops.GATE_BLOCK)
+    assert got.shape == (m, inter) and got.dtype == dtype
+    close(got, want, 1e-5 if dtype == F32 else 8e-3, f"gated {m}x{k}->{inter}")
+    # and with the plain layout (gates, then ups) through the two-kernel path
+    close(ops.gated_linear(x, torch.cat((gate, up)).contiguous(), out_dtype=dtype), want, 1e-5 if dtype == F32 else 8e-3, "halves")
 
 
 # ------------------------------------------------------------------------------------------ matrix products
