@@ -566,30 +566,28 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
 // ---------------------------------------------------------------------------------------------
 // Gated feed-forward input for few rows (M <= 16): out[m, i] = silu(x . gate_i) * (x . up_i), bf16
 // [M, inter], from W [2 inter, K] that holds alternating blocks of 16 gate rows and 16 up rows. One
-// block of 4 waves per 16 outputs: wave w takes K slabs w, w + 4, ... of the 32 weight rows (their
-// loads all in flight at once), the four partial results meet in LDS and wave 0 adds them in wave
-// order, applies the activation and stores. No partial sums leave the block and no second kernel
-// runs. K must be a multiple of 256 and rows 16-byte aligned.
-__global__ __launch_bounds__(256) void gemm_bf16_small_gated_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+// block of 8 waves per 16 outputs: waves 0-3 take the gate rows, waves 4-7 the up rows, wave w of each
+// four the K slabs w, w + 4, ... (one slab each up to K = 1024: all loads of the block in flight at
+// once, 8 KB per wave as in the split product). The eight partial results meet in LDS and wave 0 adds
+// them in wave order, applies the activation and stores. No partial sums leave the block and no
+// second kernel runs. K must be a multiple of 256 and rows 16-byte aligned.
+__global__ __launch_bounds__(512) void gemm_bf16_small_gated_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                     bf16* __restrict__ out, int M, int inter, int K,
                                                                     int ldx) {
-  __shared__ float red[4][2][WAVE][4];
+  __shared__ float red[8][WAVE][4];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int nb = blockIdx.x * 32;  // first weight row of the pair of blocks
-  floatx4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
-  const bf16* wg = W + (size_t)(nb + r) * K + g * 16;
-  const bf16* wu = wg + (size_t)16 * K;
+  const int nb = blockIdx.x * 32 + (wave / 4) * 16;  // first weight row of this wave's block of 16
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bf16* wp = W + (size_t)(nb + r) * K + g * 16;
   const bf16* xp = X + (size_t)min(r, M - 1) * ldx + g * 16;  // rows beyond M: read row M - 1, use zeros
   const uint4 zero = make_uint4(0, 0, 0, 0);
-  for (int k0 = wave * SMALL_SLAB; k0 < K; k0 += 4 * SMALL_SLAB) {
-    Chunk a[SMALL_SLAB / 64][2], b[SMALL_SLAB / 64][2], x[SMALL_SLAB / 64][2];
+  for (int k0 = (wave % 4) * SMALL_SLAB; k0 < K; k0 += 4 * SMALL_SLAB) {
+    Chunk a[SMALL_SLAB / 64][2], x[SMALL_SLAB / 64][2];
 #pragma unroll
     for (int u = 0; u < SMALL_SLAB / 64; ++u) {
-      a[u][0].u = *reinterpret_cast<const uint4*>(wg + k0 + u * 64);
-      a[u][1].u = *reinterpret_cast<const uint4*>(wg + k0 + u * 64 + 8);
-      b[u][0].u = *reinterpret_cast<const uint4*>(wu + k0 + u * 64);
-      b[u][1].u = *reinterpret_cast<const uint4*>(wu + k0 + u * 64 + 8);
+      a[u][0].u = *reinterpret_cast<const uint4*>(wp + k0 + u * 64);
+      a[u][1].u = *reinterpret_cast<const uint4*>(wp + k0 + u * 64 + 8);
     }
 #pragma unroll
     for (int u = 0; u < SMALL_SLAB / 64; ++u) {
@@ -600,17 +598,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_gated_kernel(const bf16* 
     }
 #pragma unroll
     for (int u = 0; u < SMALL_SLAB / 64; ++u) {
-      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][0].v, x[u][0].v, acc_g, 0, 0, 0);
-      acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][0].v, x[u][0].v, acc_u, 0, 0, 0);
-      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][1].v, x[u][1].v, acc_g, 0, 0, 0);
-      acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][1].v, x[u][1].v, acc_u, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][0].v, x[u][0].v, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][1].v, x[u][1].v, acc, 0, 0, 0);
     }
   }
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    red[wave][0][lane][e] = acc_g[e];
-    red[wave][1][lane][e] = acc_u[e];
-  }
+  for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
   __syncthreads();
   if (wave != 0 || r >= M) return;
   // This lane: outputs 16 blockIdx.x + 4 g + e of row m = r.
@@ -620,8 +613,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_gated_kernel(const bf16* 
     float gate = 0.f, up = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      gate += red[w][0][lane][e];
-      up += red[w][1][lane][e];
+      gate += red[w][lane][e];
+      up += red[4 + w][lane][e];
     }
     o.e[e] = static_cast<bf16>(gate / (1.f + expf(-gate)) * up);
   }
@@ -642,7 +635,7 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
   const int N = 2 * inter;
   if (M <= 16) {
     if (K % SMALL_SLAB || K / SMALL_SLAB > 8) return MS_UNSUPPORTED;
-    gemm_bf16_small_gated_kernel<<<inter / 16, 256, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    gemm_bf16_small_gated_kernel<<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
     return launch_status();
   }
   if (M <= 64 || K % BK) return MS_UNSUPPORTED;
