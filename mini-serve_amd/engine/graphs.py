@@ -13,6 +13,9 @@ The logits come back as a view of the graph's static output, valid until the nex
 
 from __future__ import annotations
 
+import gc
+import weakref
+
 import numpy as np
 import torch
 
@@ -35,7 +38,9 @@ class DecodeGraphs:
     MIN_WIDTH = 16
 
     def __init__(self, runner, max_bs: int):
-        self.runner = runner
+        # No cycle with the runner: the graphs must go when the runner goes, not whenever the cyclic
+        # collector gets to them (which may be in the middle of another runner's capture).
+        self.runner = weakref.proxy(runner)
         self.buckets = graph_buckets(max_bs)
         self.max_bs = max_bs
         self.captured: dict = {}
@@ -103,8 +108,16 @@ class DecodeGraphs:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         c.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(c.graph, pool=self.pool):
-            c.logits = model.forward(b, pool)
+        # The cyclic collector stays off while the stream is capturing: what it might free then (a
+        # graph, a stream, an event of some earlier object) may not be freed during a capture.
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(c.graph, pool=self.pool):
+                c.logits = model.forward(b, pool)
+        finally:
+            if collecting:
+                gc.enable()
         if self.pool is None:
             self.pool = c.graph.pool()
         return c
