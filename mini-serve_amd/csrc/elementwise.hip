@@ -411,7 +411,7 @@ struct Vec8<float> {
   }
 };
 
-template <typename T, typename TW, int D>
+template <typename T, typename TW, int D, int HPB>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_tile_kernel(
     const T* qkv, const float* __restrict__ parts, int splits, size_t split_stride, T* q_out, int q_out_stride,
     const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
@@ -420,107 +420,135 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_tile_kernel(
   constexpr int TOK = 256 / TPT;  // tokens per block
   constexpr int RUNS = TOK / 8;   // runs of 8 tokens
   __shared__ __attribute__((aligned(16))) T vt[TOK][D + 8];
-  const int hs = blockIdx.y;
-  const int kind = hs < Hq ? 0 : (hs < Hq + Hkv ? 1 : 2);  // the same for the whole block
+  // blockIdx.y walks groups of up to HPB heads of one kind: query groups, then key groups, then value
+  // groups. A thread loads its 8 elements of every head of the group before it works on any (HPB
+  // loads in flight), and the rotation's cosines and sines once for all of them.
+  const int nq = (Hq + HPB - 1) / HPB, nk = (Hkv + HPB - 1) / HPB;
+  int kind, h0, of_kind;
+  if ((int)blockIdx.y < nq) { kind = 0; h0 = blockIdx.y * HPB; of_kind = Hq; }
+  else if ((int)blockIdx.y < nq + nk) { kind = 1; h0 = (blockIdx.y - nq) * HPB; of_kind = Hkv; }
+  else { kind = 2; h0 = (blockIdx.y - nq - nk) * HPB; of_kind = Hkv; }
+  const int hn = min(HPB, of_kind - h0);                           // heads of this block
+  const int hs0 = (kind == 0 ? 0 : (kind == 1 ? Hq : Hq + Hkv)) + h0;  // its first head slot
   const int tl = threadIdx.x / TPT, i = threadIdx.x % TPT;
   const int t0 = blockIdx.x * TOK, t = t0 + tl;
   const bool live = t < tokens;
-  const size_t at = ((size_t)(live ? t : tokens - 1) * (Hq + 2 * Hkv) + hs) * D + i * 8;
+  const size_t at0 = ((size_t)(live ? t : tokens - 1) * (Hq + 2 * Hkv) + hs0) * D + i * 8;
 
-  float x[8];
-  if (parts != nullptr) {
+  float x[HPB][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = 0.f;
-    for (int s0 = 0; s0 < splits; s0 += 4) {  // ascending split order; the loads of four splits go out together
-      float4 a[4], b[4];
+  for (int h = 0; h < HPB; ++h) {
+    const size_t at = at0 + (size_t)(h < hn ? h : 0) * D;
+    if (parts != nullptr) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const bool in = s0 + u < splits;
-        const float* src = parts + (size_t)(in ? s0 + u : 0) * split_stride + at;
-        a[u] = *reinterpret_cast<const float4*>(src);
-        b[u] = *reinterpret_cast<const float4*>(src + 4);
-        if (!in) a[u] = b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int e = 0; e < 8; ++e) x[h][e] = 0.f;
+      for (int s0 = 0; s0 < splits; s0 += 4) {  // ascending split order; the loads of four splits go out together
+        float4 a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const bool in = s0 + u < splits;
+          const float* src = parts + (size_t)(in ? s0 + u : 0) * split_stride + at;
+          a[u] = *reinterpret_cast<const float4*>(src);
+          b[u] = *reinterpret_cast<const float4*>(src + 4);
+          if (!in) a[u] = b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          x[h][0] += a[u].x; x[h][1] += a[u].y; x[h][2] += a[u].z; x[h][3] += a[u].w;
+          x[h][4] += b[u].x; x[h][5] += b[u].y; x[h][6] += b[u].z; x[h][7] += b[u].w;
+        }
       }
+    } else {
+      Vec8<T> v;
+      v.load(qkv + at);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        x[0] += a[u].x; x[1] += a[u].y; x[2] += a[u].z; x[3] += a[u].w;
-        x[4] += b[u].x; x[5] += b[u].y; x[6] += b[u].z; x[7] += b[u].w;
-      }
+      for (int e = 0; e < 8; ++e) x[h][e] = v.get(e);
     }
-  } else {
-    Vec8<T> v;
-    v.load(qkv + at);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = v.get(e);
   }
 
   if (kind != 2) {
     const TW* w = kind == 0 ? qw : kw;
+    float wv[8], c[8], sn[8];
     if (w != nullptr) {
-      float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
-#pragma unroll
-      for (int o = 1; o < TPT; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
-      const float rstd = rsqrtf(ss / (float)D + eps);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = x[e] * rstd * to_f32(w[i * 8 + e]);
+      for (int e = 0; e < 8; ++e) wv[e] = to_f32(w[i * 8 + e]);
     }
     if (rope != nullptr) {
       const int j0 = (i % (TPT / 2)) * 8;
       const float* cs = rope + (size_t)(live ? t : tokens - 1) * D + j0;
       const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
       const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2), s1 = *reinterpret_cast<const float4*>(cs + D / 2 + 4);
-      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-      const bool low = i < TPT / 2;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float partner = __shfl_xor(x[e], TPT / 2, WAVE);
-        x[e] = low ? x[e] * c[e] - partner * sn[e] : x[e] * c[e] + partner * sn[e];
-      }
+      c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+      sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
     }
-    if (live) {
-      Vec8<T> v;
+    const bool low = i < TPT / 2;
+    const int slot = (kind == 1 && live) ? slots[t] : 0;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v.set(e, x[e]);
-      if (kind == 0) {
-        v.store(q_out + (size_t)t * q_out_stride + (size_t)hs * D + i * 8);
-      } else {
-        const int s = slots[t];
-        v.store(kc + (((size_t)(s / page_size) * Hkv + (hs - Hq)) * page_size + (s % page_size)) * D + i * 8);
+    for (int h = 0; h < HPB; ++h) {
+      if (h >= hn) break;  // the same for the whole block
+      if (w != nullptr) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[h][e] * x[h][e];
+#pragma unroll
+        for (int o = 1; o < TPT; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+        const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[h][e] = x[h][e] * rstd * wv[e];
+      }
+      if (rope != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float partner = __shfl_xor(x[h][e], TPT / 2, WAVE);
+          x[h][e] = low ? x[h][e] * c[e] - partner * sn[e] : x[h][e] * c[e] + partner * sn[e];
+        }
+      }
+      if (live) {
+        Vec8<T> v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v.set(e, x[h][e]);
+        if (kind == 0) {
+          v.store(q_out + (size_t)t * q_out_stride + (size_t)(h0 + h) * D + i * 8);
+        } else {
+          v.store(kc + (((size_t)(slot / page_size) * Hkv + (h0 + h)) * page_size + (slot % page_size)) * D + i * 8);
+        }
       }
     }
     return;
   }
 
-  // Value head: through LDS, then thread (d, run) writes tokens 8 run .. 8 run + 7 of head element d.
-  {
-    Vec8<T> v;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v.set(e, x[e]);
-    v.store(&vt[tl][i * 8]);
-  }
-  __syncthreads();
+  // Value heads: through LDS, then thread (d, run) writes tokens 8 run .. 8 run + 7 of head element d.
   const int d = threadIdx.x / RUNS, run = threadIdx.x % RUNS;
   const int tr = t0 + run * 8;
-  if (tr >= tokens) return;
-  const int kvh = hs - Hq - Hkv;
   const int n_live = min(8, tokens - tr);
   int sl[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) sl[e] = slots[min(tr + e, tokens - 1)];
+  for (int e = 0; e < 8; ++e) sl[e] = slots[max(0, min(tr + e, tokens - 1))];
   bool run_ok = n_live == 8 && (page_size % 8 == 0) && (sl[0] % 8 == 0);
 #pragma unroll
   for (int e = 1; e < 8; ++e) run_ok = run_ok && sl[e] == sl[0] + e;
-  if (run_ok) {
-    Vec8<T> v;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v.set(e, to_f32(vt[run * 8 + e][d]));
-    v.store(vc + (((size_t)(sl[0] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[0] % page_size));
-  } else {
-    for (int e = 0; e < n_live; ++e)
-      vc[(((size_t)(sl[e] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[e] % page_size)] = vt[run * 8 + e][d];
+  for (int h = 0; h < HPB; ++h) {
+    if (h >= hn) break;  // the same for the whole block
+    if (h > 0) __syncthreads();  // the previous head has been read out
+    {
+      Vec8<T> v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v.set(e, x[h][e]);
+      v.store(&vt[tl][i * 8]);
+    }
+    __syncthreads();
+    if (tr >= tokens) continue;
+    const int kvh = h0 + h;
+    if (run_ok) {
+      Vec8<T> v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v.set(e, to_f32(vt[run * 8 + e][d]));
+      v.store(vc + (((size_t)(sl[0] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[0] % page_size));
+    } else {
+      for (int e = 0; e < n_live; ++e)
+        vc[(((size_t)(sl[e] / page_size) * Hkv + kvh) * D + d) * page_size + (sl[e] % page_size)] = vt[run * 8 + e][d];
+    }
   }
 }
 
@@ -546,14 +574,20 @@ extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int sp
                      (parts == nullptr || split_stride % 4 == 0);
   if (tiled) {
     const int tok_per_block = 256 / (D / 8);
-    const dim3 grid((tokens + tok_per_block - 1) / tok_per_block, heads);
-#define LAUNCH_TILE(T, TW, DD)                                                                                          \
-  qk_norm_rope_store_tile_kernel<T, TW, DD><<<grid, 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride,   \
-                                                                   (T*)q_out, q_out_stride, slots, (const TW*)qw,        \
-                                                                   (const TW*)kw, eps, rope, (T*)kc, (T*)vc, tokens, Hq, \
-                                                                   Hkv, page_size)
-#define LAUNCH_TILE_D(T, TW) \
-  if (D == 128) LAUNCH_TILE(T, TW, 128); else LAUNCH_TILE(T, TW, 64)
+    // Many tokens: four heads of a kind per block (more loads in flight per thread, the rotation's
+    // cosines and sines read once for the four). Few tokens: a block per head, for more blocks.
+    const int hpb = tokens > 256 ? 4 : 1;
+    const dim3 grid((tokens + tok_per_block - 1) / tok_per_block, (Hq + hpb - 1) / hpb + (slots ? 2 * ((Hkv + hpb - 1) / hpb) : 0));
+#define LAUNCH_TILE(T, TW, DD, HH)                                                                                       \
+  qk_norm_rope_store_tile_kernel<T, TW, DD, HH><<<grid, 256, 0, st>>>((const T*)qkv, parts, splits, (size_t)split_stride, \
+                                                                       (T*)q_out, q_out_stride, slots, (const TW*)qw,     \
+                                                                       (const TW*)kw, eps, rope, (T*)kc, (T*)vc, tokens,  \
+                                                                       Hq, Hkv, page_size)
+#define LAUNCH_TILE_D(T, TW)                                                 \
+  if (D == 128 && hpb == 4) LAUNCH_TILE(T, TW, 128, 4);                      \
+  else if (D == 128) LAUNCH_TILE(T, TW, 128, 1);                             \
+  else if (hpb == 4) LAUNCH_TILE(T, TW, 64, 4);                              \
+  else LAUNCH_TILE(T, TW, 64, 1)
     if (is_bf16 && w_is_bf16) { LAUNCH_TILE_D(bf16, bf16); }
     else if (is_bf16) { LAUNCH_TILE_D(bf16, float); }
     else if (w_is_bf16) { LAUNCH_TILE_D(float, bf16); }

@@ -270,8 +270,9 @@ def test_rope_table(ops):
 
 
 # (tokens, layout of the slots): few tokens run the kernel with a wave per head, many the tiled one,
-# whose value store takes whole aligned runs of a page with one vector and everything else singly.
-QK_CASES = [(11, "scattered"), (150, "scattered"), (150, "runs"), (200, "shifted")]
+# whose value store takes whole aligned runs of a page with one vector and everything else singly; above
+# 256 tokens a block of the tiled kernel takes four heads of a kind.
+QK_CASES = [(11, "scattered"), (150, "scattered"), (150, "runs"), (200, "shifted"), (300, "runs"), (333, "shifted")]
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -282,7 +283,7 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page, t, layout):
     pages, eps = (t + page - 1) // page + 9, 1e-5
     qkv = rand((t, (hq + 2 * hkv) * d), dtype, 16)
     qw, kw = rand((d,), dtype, 17) + 1, rand((d,), dtype, 18) + 1
-    pos = torch.tensor(([0, 1, 2, 3, 40, 41, 700, 5, 6, 7, 4000] * 20)[:t], dtype=torch.int32, device=DEV)
+    pos = torch.tensor(([0, 1, 2, 3, 40, 41, 700, 5, 6, 7, 4000] * 40)[:t], dtype=torch.int32, device=DEV)
     if layout == "scattered":
         perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(1))[:t]
     elif layout == "runs":  # consecutive slots from a page's start, as a prompt's portion has them
