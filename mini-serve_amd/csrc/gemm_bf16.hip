@@ -191,10 +191,27 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+struct TileId {
+  int m, n, split;
+};
+
+// Block `block` of a one-dimensional grid over splits x row tiles x column tiles. Column tiles run
+// fastest, then row tiles, inside bands of `band_cols` column tiles: the blocks that run together share
+// a row of activations and, band_cols being a multiple of the eight XCDs that blocks are handed to in
+// turn, every weight tile column stays with one XCD's L2; the band bounds how much weight memory is
+// live until all row tiles have used it, so that it stays in the last-level cache.
+__device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int col_tiles, int band_cols) {
+  const int tiles = row_tiles * col_tiles;
+  const int t = block % tiles;
+  const int band = t / (band_cols * row_tiles), w = t % (band_cols * row_tiles);
+  const int cols = min(band_cols, col_tiles - band * band_cols);
+  return TileId{w / cols, band * band_cols + w % cols, block / tiles};
+}
+
 template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
 __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
-                                                               int ldx, int ldc, int k_per, size_t c_split_stride) {
+                                                               int ldx, int ldc, int k_per, size_t c_split_stride, int band_cols) {
   constexpr int WM = BM / 2, WN = BN / 2;
   constexpr int FM = WM / 16, FN = WN / 16;
   constexpr int ROW_BYTES = KS * 2;           // a tile row: KS k of bf16
@@ -206,12 +223,13 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
 
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const TileId id = tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, band_cols);
+  const int m0 = id.m * BM, n0 = id.n * BN;
   const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
-  const int k_lo = blockIdx.z * k_per;
+  const int k_lo = id.split * k_per;
   const int K = min(Kfull, k_lo + k_per);
   const int slabs = (K - k_lo) / KS;
-  void* C = mode == 1 ? (void*)((float*)Cbase + blockIdx.z * c_split_stride) : Cbase;
+  void* C = mode == 1 ? (void*)((float*)Cbase + id.split * c_split_stride) : Cbase;
 
   // Load side: instruction j of this wave fills tile rows (wave * XI + j) * 8 .. + 7.
   const int lrow = lane / CPR, lslot = lane % CPR;
@@ -466,6 +484,11 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
   return launch_status();
 }
 
+// Weight memory that one band of tile columns may span: well inside the 256 MB last-level cache. Without
+// bands the 32B gate/up product (524 MB of weights, re-read by each of 16 row tiles) ran at 650 TFLOP/s,
+// bound by memory; with them at 850-950.
+constexpr long DMA_BAND_BYTES = 96L << 20;
+
 template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
 static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
                       size_t stride, int splits, hipStream_t st) {
@@ -477,9 +500,17 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
       return MS_LAUNCH_FAILED;
     ready = true;
   }
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits);
-  if (grid.y > 65535) return MS_BAD_ARG;
-  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<grid, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride);
+  const long blocks = (long)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
+  if (blocks > 0x7fffffffL) return MS_BAD_ARG;
+  // Weight tile columns of a band: what fits in DMA_BAND_BYTES but at least 32 (four per XCD: with fewer,
+  // many blocks of an XCD wait for the same slab at the same time, which measured slower than no bands),
+  // then evened out over the bands and rounded to a multiple of eight.
+  const int col_tiles = (N + BN - 1) / BN;
+  long band_cols = DMA_BAND_BYTES / ((long)BN * K * 2);
+  if (band_cols < 32) band_cols = 32;
+  const long bands = (col_tiles + band_cols - 1) / band_cols;
+  band_cols = ((col_tiles + bands - 1) / bands + 7) / 8 * 8;
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<(unsigned)blocks, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, (int)band_cols);
   return launch_status();
 }
 
