@@ -336,28 +336,34 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
 // ---------------------------------------------------------------------------------------------
 // Small-M kernel: M <= 16 * MB rows of X (a decode step). Pure weight streaming: a wave owns 16 weight
 // rows and a slice of K; per step of 64 k each lane loads 32 bytes of its weight row and issues two
-// MFMAs per 16-row block of X. With MB == 1 the matching 32 bytes of an X row come straight from
-// global memory (X is a few KB and stays in the vector cache; no LDS, no barrier); with MB > 1 the
-// block's four waves stage the X slab of their common K slice in LDS. K is split over the grid so
+// MFMAs per 16-row block of X. Without SHARED (MB == 1 only) the matching 32 bytes of an X row come
+// straight from global memory (no LDS, no barrier: the cheapest form where launch and latency decide);
+// with SHARED the block's four waves stage the X slab of their common K slice in LDS, so that X passes
+// through the caches once per 64 weight rows instead of once per 16 (it is half the weights' bytes at
+// 8 rows, and what then limits large matrices). K is split over the grid so
 // that even a 1024-row matrix gives every CU several waves; each split writes float partial sums
 // P[split, M, N], which the caller's next kernel (or the reduction below) sums in ascending split
 // order. The number of splits depends on N, K and on whether M is above 16, not on M itself: a row's
 // result does not depend on the batch it is in (within the same MB).
 #define SMALL_SLAB 256  // k per iteration: four steps of 64
 #define XS_STRIDE (SMALL_SLAB + 8)
+// Up to 16 rows: the shared X slab is used from this many rows and this many weights on (measured:
+// 8 to 20 % faster at 8 to 16 rows and 8B / 32B layer shapes, slower below 4 M weights).
+constexpr int SMALL_SHARED_MIN_ROWS = 4;
+constexpr long SMALL_SHARED_MIN_WEIGHTS = 16L << 20;
 
-template <int MB>
+template <int MB, bool SHARED>
 __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                               float* __restrict__ P, int M, int N, int K, int ldx,
                                                               int steps_per_split, int splits) {
-  __shared__ __attribute__((aligned(16))) bf16 xs[MB > 1 ? MB * 16 * XS_STRIDE : 8];
+  __shared__ __attribute__((aligned(16))) bf16 xs[SHARED ? MB * 16 * XS_STRIDE : 8];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
   // The split index runs fastest over the grid: blocks that are resident together read neighbouring
   // k ranges of the same weight rows, which together are whole rows, instead of the same k range of
   // rows that lie a power of two apart (those would queue up on a few memory channels).
   const int split = blockIdx.x % splits, row_block = blockIdx.x / splits;
-  const int nb = (row_block * (blockDim.x / WAVE) + wave) * 16;  // MB == 1 runs one wave per block
+  const int nb = (row_block * (blockDim.x / WAVE) + wave) * 16;  // without a shared slab: one wave per block
   const int n = nb + r;
   const int k_begin = split * steps_per_split * 64;
   const int k_end = min(K, k_begin + steps_per_split * 64);
@@ -373,11 +379,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
     // beyond k_end are asked for at K, where load_chunk yields zeros. A slab that lies wholly inside
     // the matrix is loaded without any test, so that all its loads go out back to back.
     const bool whole = k0 + SMALL_SLAB <= k_end;
-    // MB > 1: this thread's share of the X slab goes out first (it comes from the cache and is back
+    // Shared slab: this thread's share of the X slab goes out first (it comes from the cache and is back
     // while the weights are still on their way), so that staging it in LDS costs no waiting of its own.
-    constexpr int XPT = MB > 1 ? MB * 16 * (SMALL_SLAB / 8) / 256 : 1;  // 16-byte chunks per thread
+    constexpr int XPT = SHARED ? MB * 16 * (SMALL_SLAB / 8) / 256 : 1;  // 16-byte chunks per thread
     Chunk xr[XPT];
-    if (MB > 1) {
+    if (SHARED) {
       if (vecx && whole) {
         const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
@@ -412,7 +418,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
         w[u][1] = load_chunk(W, n, N, kw + 8, K, K, vecw);
       }
     }
-    if (MB == 1) {
+    if (!SHARED) {
+      static_assert(SHARED || MB == 1, "more than 16 rows need the shared slab");
       Chunk x[SMALL_SLAB / 64][2];
       if (vecx && whole) {
         const bf16* xp = X + (size_t)min(r, M - 1) * ldx + k0 + g * 16;  // rows beyond M: read row M - 1, use zeros
@@ -584,9 +591,12 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   const bf16* w = (const bf16*)W;
   // Without a shared X slab the waves of a block have nothing in common: single-wave blocks spread
   // evenly over the CUs.
-  if (M <= 16) gemm_bf16_small_kernel<1><<<(unsigned)wave_blocks, WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
-  else if (M <= 32) gemm_bf16_small_kernel<2><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
-  else gemm_bf16_small_kernel<4><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  // evenly over the CUs. Both forms add up the same products in the same order.
+  const bool shared = M >= SMALL_SHARED_MIN_ROWS && (long)N * K >= SMALL_SHARED_MIN_WEIGHTS;
+  if (M <= 16 && !shared) gemm_bf16_small_kernel<1, false><<<(unsigned)wave_blocks, WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  else if (M <= 16) gemm_bf16_small_kernel<1, true><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  else if (M <= 32) gemm_bf16_small_kernel<2, true><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
+  else gemm_bf16_small_kernel<4, true><<<(unsigned)wide_blocks, 256, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
   if (reduce) {
     if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;
     splitk_reduce_kernel<<<dim3((N + 255) / 256, M), 256, 0, st>>>(partials, C, mode, splits, M, N, ldc);

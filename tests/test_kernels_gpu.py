@@ -222,6 +222,24 @@ def test_pending_sums_feed_their_consumers(ops, m):
     close(r4, full, 1e-5, "accumulate")
 
 
+@pytest.mark.parametrize("n,k", [(4112, 4096), (33000, 520)])
+def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
+    """Above 16 M weights and from 4 rows on, the product for up to 16 rows stages its rows in LDS for
+    four waves (N no multiple of 64: the last block has waves without weight rows; K = 520: a slab that
+    is cut off). Both forms add the same products in the same order: a row gives the same bits alone."""
+    x, w = rand((16, k), BF16, 70), rand((n, k), BF16, 71, 0.05)
+    want = x.double() @ w.double().T
+    rows = {}
+    for m in (1, 3, 4, 9, 16):
+        s = ops.linear(x[:m].contiguous(), w, out_dtype=BF16, defer=True)
+        assert isinstance(s, ops.SplitSum)
+        rows[m] = s.parts.clone()
+        close(rows[m].sum(0), want[:m], 1e-5, f"{m} rows of {n}x{k}")
+    for m in (3, 4, 9, 16):
+        assert torch.equal(rows[m][:, :1], rows[1])
+    assert torch.equal(rows[16][:, :9], rows[9])
+
+
 @pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 4), (2048, 1024, 3072, 2), (300, 1000, 1100, 2), (2048, 4096, 1024, 1)])
 def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
     x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
