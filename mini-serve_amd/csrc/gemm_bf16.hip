@@ -195,23 +195,47 @@ struct TileId {
   int m, n, split;
 };
 
-// Block `block` of a one-dimensional grid over splits x row tiles x column tiles. Column tiles run
-// fastest, then row tiles, inside bands of `band_cols` column tiles: the blocks that run together share
-// a row of activations and, band_cols being a multiple of the eight XCDs that blocks are handed to in
-// turn, every weight tile column stays with one XCD's L2; the band bounds how much weight memory is
-// live until all row tiles have used it, so that it stays in the last-level cache.
-__device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int col_tiles, int band_cols) {
+// Tile `t` of a grid of rows x cols tiles: column tiles run fastest, then row tiles, inside bands of
+// `band_cols` column tiles. The blocks that run together share a row of activations; the band bounds
+// how much weight memory is live until all row tiles have used it, so that it stays in the last-level
+// cache.
+__device__ __forceinline__ void banded(int t, int rows, int cols, int band_cols, int& m, int& n) {
+  const int band = t / (band_cols * rows), w = t % (band_cols * rows);
+  const int width = min(band_cols, cols - band * band_cols);
+  m = w / width;
+  n = band * band_cols + w % width;
+}
+
+// Block `block` of a one-dimensional grid over splits x row tiles x column tiles. Blocks are handed to
+// the eight XCDs in turn (block L to XCD L % 8), each with an L2 of its own. With xcd_rows == 0 the
+// tiles are walked in banded order over the whole grid: band_cols being a multiple of eight, a weight
+// tile column stays with one XCD, and every XCD reads all activations. With xcd_rows = 2, 4 or 8 (the
+// caller has checked that the tile counts divide) the XCDs form a grid of xcd_rows x 8 / xcd_rows, each
+// owning a rectangle of tiles that it walks in banded order: then an XCD reads only its share of the
+// activations, which is what counts when the weight matrix is the smaller operand.
+__device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int col_tiles, int xcd_rows, int band_cols) {
   const int tiles = row_tiles * col_tiles;
   const int t = block % tiles;
-  const int band = t / (band_cols * row_tiles), w = t % (band_cols * row_tiles);
-  const int cols = min(band_cols, col_tiles - band * band_cols);
-  return TileId{w / cols, band * band_cols + w % cols, block / tiles};
+  TileId id;
+  id.split = block / tiles;
+  if (xcd_rows == 0) {
+    banded(t, row_tiles, col_tiles, band_cols, id.m, id.n);
+    return id;
+  }
+  const int xcd_cols = 8 / xcd_rows;
+  const int xcd = t % 8, slot = t / 8;
+  const int sub_rows = row_tiles / xcd_rows, sub_cols = col_tiles / xcd_cols;
+  banded(slot, sub_rows, sub_cols, band_cols, id.m, id.n);
+  id.m += (xcd / xcd_cols) * sub_rows;
+  id.n += (xcd % xcd_cols) * sub_cols;
+  return id;
 }
 
 template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
 __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
-                                                               int ldx, int ldc, int k_per, size_t c_split_stride, int band_cols) {
+                                                               int ldx, int ldc, int k_per, size_t c_split_stride, int xcd_rows,
+                                                               int band_cols) {
   constexpr int WM = BM / 2, WN = BN / 2;
   constexpr int FM = WM / 16, FN = WN / 16;
   constexpr int ROW_BYTES = KS * 2;           // a tile row: KS k of bf16
@@ -223,7 +247,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
 
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const TileId id = tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, band_cols);
+  const TileId id = tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, xcd_rows, band_cols);
   const int m0 = id.m * BM, n0 = id.n * BN;
   const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
   const int k_lo = id.split * k_per;
@@ -509,15 +533,39 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
   }
   const long blocks = (long)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
   if (blocks > 0x7fffffffL) return MS_BAD_ARG;
-  // Weight tile columns of a band: what fits in DMA_BAND_BYTES but at least 32 (four per XCD: with fewer,
-  // many blocks of an XCD wait for the same slab at the same time, which measured slower than no bands),
-  // then evened out over the bands and rounded to a multiple of eight.
-  const int col_tiles = (N + BN - 1) / BN;
+  // How the XCDs share the tiles: as a grid of xcd_rows x 8 / xcd_rows rectangles where the tile counts
+  // divide, chosen so that the bytes all XCDs read together (its share of the activations once per
+  // XCD column, its share of the weights once per XCD row) are fewest, if that is under 0.6 of what
+  // columns in turn (0) read: measured, a smaller advantage does not pay (N = 1024 at 2,048 rows: 10 %
+  // faster; N = 4096 to 6144: 2 to 5 % slower).
+  const int row_tiles = (M + BM - 1) / BM, col_tiles = (N + BN - 1) / BN;
+  int xcd_rows = 0;
+  long least = (8L * M + N) * 6 / 10;
+  for (int pm = 2; pm <= 8; pm *= 2) {
+    const int pn = 8 / pm;
+    if (row_tiles % pm || col_tiles % pn) continue;
+    const long cost = (long)pn * M + (long)pm * N;
+    if (cost < least) {
+      least = cost;
+      xcd_rows = pm;
+    }
+  }
+  // Weight tile columns of a band: what fits in DMA_BAND_BYTES but at least 32 over all XCDs (four per
+  // XCD: with fewer, many blocks of an XCD wait for the same slab at the same time, which measured
+  // slower than no bands), then evened out over the bands; a multiple of eight where the XCDs take
+  // columns in turn.
   long band_cols = DMA_BAND_BYTES / ((long)BN * K * 2);
   if (band_cols < 32) band_cols = 32;
-  const long bands = (col_tiles + band_cols - 1) / band_cols;
-  band_cols = ((col_tiles + bands - 1) / bands + 7) / 8 * 8;
-  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<(unsigned)blocks, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, (int)band_cols);
+  if (xcd_rows == 0) {
+    const long bands = (col_tiles + band_cols - 1) / band_cols;
+    band_cols = ((col_tiles + bands - 1) / bands + 7) / 8 * 8;
+  } else {
+    const int sub_cols = col_tiles / (8 / xcd_rows);
+    band_cols = band_cols / (8 / xcd_rows);
+    const long bands = (sub_cols + band_cols - 1) / band_cols;
+    band_cols = (sub_cols + bands - 1) / bands;
+  }
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<(unsigned)blocks, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, xcd_rows, (int)band_cols);
   return launch_status();
 }
 

@@ -166,11 +166,14 @@ def test_gemm_bf16(ops, m, n, k):
     close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
 
 
-@pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024)])
+@pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024),
+                                   (4000, 1500, 192), (1990, 1000, 128)])
 def test_gemm_bf16_large_tiles(ops, m, n, k):
     """Shapes with at least 256 tiles of 128 x 128 and K a multiple of 64 take the kernel whose slabs go
     straight into LDS: edge tiles in both directions (rows past the end are read from the last valid
-    row and never stored), one slab, an odd number of slabs."""
+    row and never stored), one slab, an odd number of slabs. The last two have many more rows than
+    columns and tile counts that divide by the XCD grid (2 x 4 with 128-wide tiles, 4 x 2 with 64-wide
+    ones): each XCD then owns a rectangle of tiles, with the matrix's edges in some of them."""
     x, w = rand((m, k), BF16, 14), rand((n, k), BF16, 15)
     want = x.double() @ w.double().T
     close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
