@@ -245,23 +245,21 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
     }
 #pragma unroll
     for (int b = 0; b < NQ; ++b) {
-      float m_new = m_run[b];
+      // The maximum is taken over the raw scores (the scale is positive) and scaled once; the scale
+      // itself enters in the exponent's fused multiply-add. -inf stays -inf through both.
+      float s_max = -INFINITY;
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = s[b][tb][i] * scale2;  // -inf stays -inf (the scale is positive)
-          s[b][tb][i] = v;
-          m_new = fmaxf(m_new, v);
-        }
-      m_new = rows4_max(m_new);
+        for (int i = 0; i < 4; ++i) s_max = fmaxf(s_max, s[b][tb][i]);
+      const float m_new = fmaxf(m_run[b], rows4_max(s_max) * scale2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
       float psum = 0.f;
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = __builtin_amdgcn_exp2f(s[b][tb][i] - m_safe);
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][tb][i], scale2, -m_safe));
           psum += p;
           pf[b][tb / 2][(tb % 2) * 4 + i] = static_cast<bf16>(p);
         }
@@ -269,10 +267,14 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
       const float corr = __builtin_amdgcn_exp2f(m_run[b] - m_safe);
       l_run[b] = l_run[b] * corr + psum;
       m_run[b] = m_new;
+      // Once the maxima of a wave's rows have settled (after the first few tiles, as a rule) the
+      // correction is exactly 1 for all of them, and the output is left alone.
+      if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[b][db][i] *= corr;  // the lane's output values are all of its own row
+          for (int i = 0; i < 4; ++i) o[b][db][i] *= corr;  // the lane's output values are all of its own row
+      }
     }
     {
       // The same for the V^T fragments of the second product: keys 8 g .. 8 g + 7 of the pair.
