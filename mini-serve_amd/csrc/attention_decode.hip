@@ -32,14 +32,81 @@ struct DecodeTile {
   bf16x8 v[D / 16];
 };
 
+// The fused form takes, instead of finished queries and a cache that already holds the new token, the
+// qkv projection as it leaves the small-M product: float partial sums [splits, tokens, (Hq + 2 Hkv) D].
+// Every wave sums, norms and rotates the queries of its KV head's group itself (a few hundred floats);
+// the one wave whose chunks end with the sequence's last token does the same for the new key, takes
+// the new value, stores both into the cache and puts them into its operands of that chunk in
+// registers (what its loads brought from the not yet written slot is replaced, so no store has to be
+// waited for). This is the work of the QK-norm / rotation / store kernel, which a step of single
+// tokens then does not launch.
+struct FusedQkv {
+  const float* parts;      // [splits, tokens, row_width]
+  int splits;
+  long long split_stride;  // floats between splits
+  int row_width;           // (Hq + 2 Hkv) D
+  const bf16* q_weight;    // [D] each, or both nullptr: no norm
+  const bf16* k_weight;
+  float eps;
+  const float* rope;       // [tokens, D]: cosines, then sines, of D / 2 angles; nullptr: no rotation
+  int store;               // 0: another layer owns the cache, the new token is already in it
+};
+
+// Four consecutive elements d0 .. d0 + 3 of a head whose D / 4 holders are neighbouring lanes (an
+// aligned group): RMSNorm over the head with weight w (if any), then rotation by the angles of
+// `rope_row` (if any), element d paired with d +- D / 2. Every lane of the wave must call this.
 template <int D>
+__device__ __forceinline__ void head_norm_rotate(float (&x)[4], int d0, const bf16* __restrict__ w, float eps,
+                                                 const float* __restrict__ rope_row) {
+  if (w != nullptr) {
+    float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+#pragma unroll
+    for (int o = 1; o < D / 4; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+    const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = x[e] * rstd * to_f32(w[d0 + e]);
+  }
+  if (rope_row != nullptr) {
+    const int j0 = d0 % (D / 2);
+    const float4 c = *reinterpret_cast<const float4*>(rope_row + j0);
+    const float4 sn = *reinterpret_cast<const float4*>(rope_row + D / 2 + j0);
+    const float cs[4] = {c.x, c.y, c.z, c.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
+    const bool low = d0 < D / 2;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float partner = __shfl_xor(x[e], D / 8, WAVE);
+      x[e] = low ? x[e] * cs[e] - partner * ss[e] : x[e] * cs[e] + partner * ss[e];
+    }
+  }
+}
+
+// Sum over the splits, in ascending order, of four floats at `at` of each split.
+__device__ __forceinline__ void sum_parts4(float (&x)[4], const float* __restrict__ parts, int splits, long long stride, size_t at) {
+  x[0] = x[1] = x[2] = x[3] = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 4) {  // the loads of four splits go out together
+    float4 a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a[u] = *reinterpret_cast<const float4*>(parts + (size_t)(s0 + u < splits ? s0 + u : 0) * stride + at);
+      if (s0 + u >= splits) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      x[0] += a[u].x; x[1] += a[u].y; x[2] += a[u].z; x[3] += a[u].w;
+    }
+  }
+}
+
+template <int D, bool FUSED>
 __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
-    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const bf16* __restrict__ q, int q_stride, bf16* kc_rw, bf16* vc_rw,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tokens,
     const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int Hq, int Hkv, float scale, int window) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int Hq, int Hkv, float scale, int window, FusedQkv fin) {
   constexpr int KK = D / 32;  // k-steps of the score product
   constexpr int DB = D / 16;  // 16-wide blocks of the head
+  const bf16* kc = kc_rw;
+  const bf16* vc = vc_rw;
   const int G = Hq / Hkv;
   const int b = blockIdx.x / Hkv, kvh = blockIdx.x % Hkv;
   const int split = blockIdx.y, splits = gridDim.y;
@@ -59,7 +126,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
   bf16x8 qf[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
-    if (r < G) {
+    if (!FUSED && r < G) {
       qf[kk] = *reinterpret_cast<const bf16x8*>(q + (size_t)tok * q_stride + (size_t)(kvh * G + r) * D + kk * 32 + g * 8);
     } else {
 #pragma unroll
@@ -83,6 +150,10 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
   // hitting the same few memory channels (measured on the address pattern alone: 5.1 -> 5.8 TB/s).
   const int per_wave = (c_end - c_begin + 3) / 4;
   const int w_begin = c_begin + wave * per_wave, w_end = min(c_end, w_begin + per_wave);
+  // Fused form: this wave's chunks end with the sequence's last one, which holds the new token.
+  const bool has_new = FUSED && fin.store && w_begin < w_end && w_end == n_chunks;
+  __shared__ __attribute__((aligned(16))) bf16 qs[FUSED ? 4 : 1][FUSED ? 16 * D : 8];  // each wave's queries [G, D]
+  __shared__ __attribute__((aligned(16))) bf16 kv_new[FUSED ? 2 * D : 8];              // the new key, then the new value
   int p0n = 0, p1n = 0;
   auto fetch_ids = [&](int c) {
     if (c < w_end) {
@@ -110,8 +181,35 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
 #pragma unroll
     for (int db = 0; db < DB; ++db) t.v[db] = *reinterpret_cast<const bf16x8*>(v0 + (size_t)db * 16 * PAGE);
   };
-  auto multiply = [&](const DecodeTile<D>& t, int c) {
+  auto multiply = [&](DecodeTile<D>& t, int c) {
     const int t0 = lo_al + c * CHUNK;
+    if (FUSED && has_new && c == n_chunks - 1) {
+      // The new token is token j of this chunk: key row jt of page jp, that is row r_new of product a
+      // or b; and element j % 8 of the value operands of lane group 2 jp + jt / 8.
+      const int j = kv_len - 1 - t0, jp = j / PAGE, jt = j % PAGE;
+      const int r_new = jp * 8 + (jt / 8) * 4 + jt % 4;
+      const bool second = (jt / 4) & 1;
+      if (r == r_new) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const bf16x8 kn = *reinterpret_cast<const bf16x8*>(&kv_new[kk * 32 + g * 8]);
+          if (second) t.kb[kk] = kn;
+          else t.ka[kk] = kn;
+        }
+      }
+      // A chunk that ends in its first page reads that page for its second half as well (masked, but a
+      // probability of 0 does not wipe out whatever the unwritten slot happens to hold).
+      const bool twice = t0 + PAGE >= kv_len;
+      if (g % 2 == jt / 8 && (g / 2 == jp || twice)) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const bf16 vn = kv_new[D + db * 16 + r];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e == jt % 8) t.v[db][e] = vn;
+        }
+      }
+    }
     floatx4 s0 = floatx4{0.f, 0.f, 0.f, 0.f}, s1 = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
@@ -157,6 +255,57 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     int c = w_begin;
     fetch_ids(c);
     if (c < w_end) load(ta, c);
+    if (FUSED) {
+      // Queries of the group: G * D floats, four per lane and round. (The first chunk is on its way.)
+      const size_t row = (size_t)tok * fin.row_width;
+      const float* rope_row = fin.rope ? fin.rope + (size_t)tok * D : nullptr;
+      const int gd = G * D;
+      for (int base = 0; base < gd; base += 4 * WAVE) {
+        const int e0 = base + lane * 4;
+        const bool valid = e0 < gd;
+        const int ec = valid ? e0 : 0;
+        float x[4];
+        sum_parts4(x, fin.parts, fin.splits, fin.split_stride, row + (size_t)kvh * gd + ec);
+        head_norm_rotate<D>(x, ec % D, fin.q_weight, fin.eps, rope_row);
+        if (valid) {
+          bf16x4 xb;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) xb[e] = static_cast<bf16>(x[e]);
+          *reinterpret_cast<bf16x4*>(&qs[wave][ec]) = xb;
+        }
+      }
+      if (r < G) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8*>(&qs[wave][r * D + kk * 32 + g * 8]);
+      }
+      if (has_new) {
+        // The new key (lanes 0 .. D / 4 - 1) and value (lanes 32 .. 32 + D / 4 - 1): into the cache, and
+        // into LDS for this wave's last chunk.
+        const bool is_k = lane < 32, valid = lane % 32 < D / 4;
+        const int d0 = valid ? (lane % 32) * 4 : 0;
+        float x[4];
+        sum_parts4(x, fin.parts, fin.splits, fin.split_stride, row + (size_t)(is_k ? Hq + kvh : Hq + Hkv + kvh) * D + d0);
+        float xk[4] = {x[0], x[1], x[2], x[3]};
+        head_norm_rotate<D>(xk, d0, fin.k_weight, fin.eps, rope_row);
+        const int p = kv_len - 1;
+        const size_t page = (size_t)table[p / PAGE];
+        if (valid && is_k) {
+          bf16x4 xb;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) xb[e] = static_cast<bf16>(xk[e]);
+          *reinterpret_cast<bf16x4*>(&kv_new[d0]) = xb;
+          *reinterpret_cast<bf16x4*>(kc_rw + ((page * Hkv + kvh) * PAGE + p % PAGE) * D + d0) = xb;
+        }
+        if (valid && !is_k) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bf16 vb = static_cast<bf16>(x[e]);
+            kv_new[D + d0 + e] = vb;
+            vc_rw[((page * Hkv + kvh) * D + d0 + e) * PAGE + p % PAGE] = vb;
+          }
+        }
+      }
+    }
     while (c < w_end) {
       if (c + 1 < w_end) load(tb, c + 1);
       multiply(ta, c);
@@ -249,6 +398,21 @@ __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __re
 
 // rows decode tokens (tokens[i] = flat token index, or nullptr for the identity). part_o holds
 // rows * Hq * splits * D floats, part_ml rows * Hq * splits * 2 (unused when splits == 1).
+template <bool FUSED>
+static int launch_decode(const bf16* q, int q_stride, bf16* kc, bf16* vc, const int* block_table, int table_width,
+                         const int* tokens, const int* token_row, const int* pos, bf16* out, float* part_o, float* part_ml,
+                         int rows, int splits, int Hq, int Hkv, int D, float scale, int window, FusedQkv fin, hipStream_t st) {
+  dim3 grid(rows * Hkv, splits);
+#define LAUNCH(DD)                                                                                                      \
+  attn_decode_split_kernel<DD, FUSED><<<grid, 256, 0, st>>>(q, q_stride, kc, vc, block_table, table_width, tokens,      \
+                                                            token_row, pos, out, part_o, part_ml, Hq, Hkv, scale,       \
+                                                            window, fin);                                               \
+  if (splits > 1) attn_decode_reduce_kernel<DD><<<dim3(rows, Hq), DD, 0, st>>>(part_o, part_ml, tokens, out, Hq, splits)
+  if (D == 128) { LAUNCH(128); } else { LAUNCH(64); }
+#undef LAUNCH
+  return launch_status();
+}
+
 extern "C" int ms_attention_decode_bf16(const void* q, int q_stride, const void* kc, const void* vc,
                                         const int* block_table, int table_width, const int* tokens,
                                         const int* token_row, const int* pos, void* out, float* part_o, float* part_ml,
@@ -259,14 +423,37 @@ extern "C" int ms_attention_decode_bf16(const void* q, int q_stride, const void*
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || splits < 1 || splits > 65535 || window < 0 || table_width <= 0 ||
       q_stride < Hq * D || q_stride % 8 || (splits > 1 && (!part_o || !part_ml)))
     return MS_BAD_ARG;
-  dim3 grid(rows * Hkv, splits);
-#define LAUNCH(DD)                                                                                                     \
-  attn_decode_split_kernel<DD><<<grid, 256, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc,       \
-                                                     block_table, table_width, tokens, token_row, pos, (bf16*)out,    \
-                                                     part_o, part_ml, Hq, Hkv, scale, window);                         \
-  if (splits > 1)                                                                                                      \
-    attn_decode_reduce_kernel<DD><<<dim3(rows, Hq), DD, 0, st>>>(part_o, part_ml, tokens, (bf16*)out, Hq, splits)
-  if (D == 128) { LAUNCH(128); } else { LAUNCH(64); }
-#undef LAUNCH
-  return launch_status();
+  return launch_decode<false>((const bf16*)q, q_stride, (bf16*)kc, (bf16*)vc, block_table, table_width, tokens, token_row,
+                              pos, (bf16*)out, part_o, part_ml, rows, splits, Hq, Hkv, D, scale, window, FusedQkv{}, st);
+}
+
+// The same over the qkv projection's partial sums `parts` [qkv_splits, tokens, (Hq + 2 Hkv) D] (floats,
+// qkv_split_stride apart) of a step whose rows bring one token each: per-head RMSNorm of q and k with
+// bfloat16 weights [D] (both nullptr: none), rotation over the whole head by the table `rope`
+// [tokens, D] (nullptr: none), and, with store != 0, the new token's key and value written to its place
+// in the cache (its page is taken from the block table at pos).
+extern "C" int ms_attention_decode_fused_bf16(const float* parts, int qkv_splits, long long qkv_split_stride,
+                                              const void* q_weight, const void* k_weight, float eps, const float* rope,
+                                              int store, void* kc, void* vc, const int* block_table, int table_width,
+                                              const int* tokens, const int* token_row, const int* pos, void* out,
+                                              float* part_o, float* part_ml, int rows, int splits, int Hq, int Hkv, int D,
+                                              int page_size, float scale, int window, hipStream_t st) {
+  if (rows <= 0) return MS_OK;
+  if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || splits < 1 || splits > 65535 || window < 0 || table_width <= 0 ||
+      (splits > 1 && (!part_o || !part_ml)) || parts == nullptr || qkv_splits < 1 || qkv_split_stride % 4 ||
+      (q_weight == nullptr) != (k_weight == nullptr))
+    return MS_BAD_ARG;
+  FusedQkv fin;
+  fin.parts = parts;
+  fin.splits = qkv_splits;
+  fin.split_stride = qkv_split_stride;
+  fin.row_width = (Hq + 2 * Hkv) * D;
+  fin.q_weight = (const bf16*)q_weight;
+  fin.k_weight = (const bf16*)k_weight;
+  fin.eps = eps;
+  fin.rope = rope;
+  fin.store = store;
+  return launch_decode<true>(nullptr, 0, (bf16*)kc, (bf16*)vc, block_table, table_width, tokens, token_row, pos, (bf16*)out,
+                             part_o, part_ml, rows, splits, Hq, Hkv, D, scale, window, fin, st);
 }

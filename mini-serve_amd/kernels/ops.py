@@ -41,6 +41,9 @@ _SIGNATURES = {
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_void,
+                                       _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
+                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
                                   _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
@@ -422,6 +425,62 @@ def decode_splits(rows: int, num_kv_heads: int, max_kv_len: int) -> int:
     by_fill = -(-DECODE_TARGET_BLOCKS // max(1, rows * num_kv_heads))
     by_len = max(1, -(-max_kv_len // 32) // DECODE_MIN_CHUNKS)
     return max(1, min(by_fill, by_len))
+
+
+def decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim) -> bool:
+    """Whether ``decode_attention_fused`` takes this step: every row brings one token, the qkv
+    projection comes as partial sums, bfloat16 cache with 16-token pages, a head size of 64 or 128, at
+    most 16 query heads per KV head, bfloat16 norm weights (or none), rotation over the whole head (or
+    none)."""
+    return (isinstance(qkv, SplitSum) and batch.is_decode and batch.decode_tokens is None
+            and k_cache.dtype == BF16 and v_cache.dtype == BF16 and k_cache.dim() == 4 and k_cache.shape[2] == 16
+            and head_dim in (64, 128) and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16
+            and qkv.stride % 4 == 0
+            and (q_weight is None) == (k_weight is None) and (q_weight is None or (q_weight.dtype == BF16 and k_weight.dtype == BF16))
+            and (rope is None or rope.shape[1] == head_dim))
+
+
+def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v_cache, block_table, batch,
+                           num_heads, num_kv_heads, head_dim, scale, window) -> torch.Tensor:
+    """``qk_norm_rope_store`` and ``paged_attention`` of a step of single tokens in one kernel, from the
+    partial sums ``qkv`` (a ``SplitSum`` of ``[T, (Hq + 2 Hkv) D]``): the queries never go to memory,
+    and with ``store`` the new token's key and value are written to the cache by the block that uses
+    them first. Returns bfloat16 ``[T, Hq * D]``. ``decode_attention_fusable`` says when this applies."""
+    if not decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim):
+        raise ValueError("this step cannot run the fused decode attention")
+    _dev(qkv.parts, "qkv", F32, 3)
+    t = qkv.shape[0]
+    if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+        raise ValueError(f"qkv partial sums have width {qkv.shape[1]}, expected {(num_heads + 2 * num_kv_heads) * head_dim}")
+    page = _check_caches(k_cache, v_cache, BF16, num_kv_heads, head_dim)
+    if not scale > 0:
+        raise ValueError(f"the attention scale must be positive, not {scale}")
+    if q_weight is not None:
+        for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
+            _dev(w, nm, BF16, 1)
+            if w.shape[0] != head_dim:
+                raise ValueError(f"{nm} weight has {w.shape[0]} elements for head_dim {head_dim}")
+    if rope is not None:
+        _dev(rope, "rope", F32, 2)
+        if rope.shape[0] != t:
+            raise ValueError("one row of the rotation table per token is needed")
+    _dev(block_table, "block_table", I32, 2)
+    _dev(batch.token_row, "token_row", I32, 1)
+    _dev(batch.positions, "positions", I32, 1)
+    if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
+        raise ValueError("batch metadata does not match the number of tokens or rows")
+    out = torch.empty((t, num_heads * head_dim), dtype=BF16, device=qkv.parts.device)
+    splits = decode_splits(t, num_kv_heads, batch.max_kv_len)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((t * num_heads * splits * head_dim,), dtype=F32, device=out.device)
+        part_ml = torch.empty((t * num_heads * splits * 2,), dtype=F32, device=out.device)
+    _check(library().ms_attention_decode_fused_bf16(
+        qkv.parts.data_ptr(), qkv.splits, qkv.stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(rope), int(bool(store)),
+        k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], None,
+        batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml), t, splits,
+        num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_decode_fused")
+    return out
 
 
 def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window):

@@ -5,7 +5,8 @@ bias, per-head RMSNorm of q and k (one ``[head_dim]`` weight each, shared by all
 of q and k, store of k and v into the cache, causal attention in which query head ``h`` reads KV
 head ``h // (heads / kv_heads)`` with ``scale`` on the scores, output projection. Here the three
 projections are one matrix product over row-concatenated weights (as the reference's fused path
-does, miniserve/model/fused.py:204-206); norm, rotation and cache store are one kernel; the output
+does, miniserve/model/fused.py:204-206); norm, rotation and cache store are one kernel (in a step of
+single tokens they are part of the attention kernel); the output
 projection adds into the residual stream in its epilogue, or (few rows) leaves partial sums pending
 for the next norm to add.
 
@@ -74,10 +75,20 @@ class GQAttention(Mixer):
         ops = self.rt.ops
         qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
         rot = self.position.rotation(batch)
+        table = rot.table if rot is not None else None
+        if ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
+                                        self.heads, self.kv_heads, self.head_dim):
+            # a step of single tokens: norm, rotation, cache store and attention are one kernel
+            out = ops.decode_attention_fused(
+                qkv, self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps), table,
+                cache.writes, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
+                self.scale, self.window,
+            )
+            return ops.linear(out, self.o, accumulate_into=residual, defer=True)
         q = ops.qk_norm_rope_store(
             qkv, cache.slots if cache.writes else None,
             self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps),
-            rot.table if rot is not None else None,
+            table,
             cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, out_dtype=self.rt.dtype,
         )
         out = ops.paged_attention(

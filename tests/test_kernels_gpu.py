@@ -364,6 +364,7 @@ def make_batch(lens_new, starts):
     batch.row_lens, batch.row_starts_host = list(lens_new), list(starts)
     n_dec = sum(1 for n in lens_new if n == 1)
     batch.num_decode_tokens = n_dec
+    batch.is_decode = n_dec == len(lens_new)
     batch.decode_tokens = batch.prefill_tokens = None
     if 0 < n_dec < len(lens_new):
         dec, pre, t = [], [], 0
@@ -479,6 +480,74 @@ def test_decode_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost)
 )
 def test_prefill_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost):
     attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=40, boost=boost)
+
+
+@pytest.mark.parametrize(
+    "hq,hkv,d,starts,window,norm,rot",
+    [
+        (16, 8, 128, [0, 15, 16, 31, 32, 1000, 4095], 0, True, True),  # page and chunk edges, a sequence of one token
+        (16, 8, 128, [700, 3000], 0, False, True),
+        (16, 8, 128, [700, 3000, 5], 0, True, False),
+        (32, 8, 128, [5, 260, 90], 0, True, True),
+        (64, 8, 128, [513, 77], 0, True, True),
+        (16, 1, 128, [100, 33], 0, True, True),                        # sixteen query heads on one KV head
+        (14, 2, 64, [63, 64, 65, 2000, 1], 0, True, True),             # seven heads per group, head size 64
+        (6, 6, 64, [300, 40, 41, 1200], 100, True, True),              # one head per group, a window
+        (16, 8, 128, [500, 31, 2047], 33, True, True),
+        (4, 2, 128, list(range(0, 6400, 100)), 0, True, True),         # a full batch: one split
+    ],
+)
+def test_decode_attention_fused(ops, hq, hkv, d, starts, window, norm, rot):
+    """A step of single tokens from the qkv projection's partial sums in one kernel gives what the
+    norm / rotation / store kernel followed by the decode attention gives: the outputs, and the new
+    token's key and value in the cache. The new token's slots hold NaN beforehand: nothing may be read
+    from them."""
+    page, eps, b = 16, 1e-6, len(starts)
+    g = torch.Generator().manual_seed(5)
+    blocks = [-(-(s + 1) // page) for s in starts]
+    pages = sum(blocks) + 3
+    order = torch.randperm(pages, generator=g).tolist()
+    table = torch.full((b, max(blocks)), -1, dtype=torch.int32)
+    at = 0
+    for i, nb in enumerate(blocks):
+        table[i, :nb] = torch.tensor(order[at : at + nb], dtype=torch.int32)
+        at += nb
+    slots = torch.tensor([int(table[i, s // page]) * page + s % page for i, s in enumerate(starts)], dtype=torch.int32, device=DEV)
+    kc, vc = rand((pages, hkv, page, d), BF16, 81), rand((pages, hkv, d, page), BF16, 82)
+    x = rand((b, (hq + 2 * hkv) * d), BF16, 83).float()
+    parts = torch.stack([x * 0.25, x * 0.5, x * 0.125, x * 0.125, x * 0.0])  # five splits: two rounds of loads
+    qw = (rand((d,), BF16, 84) + 1) if norm else None
+    kw = (rand((d,), BF16, 85) + 1) if norm else None
+    batch = make_batch([1] * b, starts)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    rope = ops.rope_table(batch.positions, inv_freq) if rot else None
+    scale = d**-0.5
+    table = table.to(DEV)
+    assert ops.decode_attention_fusable(ops.SplitSum(parts), batch, qw, kw, rope, kc, vc, hq, hkv, d)
+
+    k1, v1 = kc.clone(), vc.clone()
+    q = ops.qk_norm_rope_store(ops.SplitSum(parts), slots, qw, kw, eps, rope, k1, v1, hq, hkv, d, out_dtype=BF16)
+    want = ops.paged_attention(q, k1, v1, table, batch, hq, hkv, d, scale, window)
+
+    k2, v2 = kc.clone(), vc.clone()
+    sl = slots.long()
+    k2[sl // page, :, sl % page] = float("nan")
+    v2[sl // page, :, :, sl % page] = float("nan")
+    assert int(torch.isnan(k2).sum()) == b * hkv * d and int(torch.isnan(v2).sum()) == b * hkv * d
+    got = ops.decode_attention_fused(ops.SplitSum(parts), qw, kw, eps, rope, True, k2, v2, table, batch, hq, hkv, d, scale, window)
+    close(got, want, 8e-3, f"fused decode attention {hq}/{hkv}/{d}")
+    flat = lambda c, v: (c.permute(0, 3, 1, 2) if v else c.permute(0, 2, 1, 3)).reshape(pages * page, hkv, d)
+    close(flat(k2, False)[sl], flat(k1, False)[sl], 8e-3, "the new keys in the cache")
+    assert torch.equal(flat(v2, True)[sl], flat(v1, True)[sl]), "the new values in the cache"
+    rest = torch.ones(pages * page, dtype=torch.bool, device=DEV)
+    rest[sl] = False
+    assert torch.equal(flat(k2, False)[rest], flat(kc, False)[rest]) and torch.equal(flat(v2, True)[rest], flat(vc, True)[rest])
+
+    # a layer that reads another layer's cache: the new token is in it already, nothing is written
+    k3, v3 = k1.clone(), v1.clone()
+    got = ops.decode_attention_fused(ops.SplitSum(parts), qw, kw, eps, rope, False, k3, v3, table, batch, hq, hkv, d, scale, window)
+    close(got, want, 8e-3, "fused decode attention without the store")
+    assert torch.equal(k3, k1) and torch.equal(v3, v1)
 
 
 def test_decode_splits_rule(ops):
