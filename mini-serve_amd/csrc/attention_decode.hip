@@ -260,6 +260,12 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
       const size_t row = (size_t)tok * fin.row_width;
       const float* rope_row = fin.rope ? fin.rope + (size_t)tok * D : nullptr;
       const int gd = G * D;
+      // The wave that holds the new token asks for its key (lanes 0 .. D / 4 - 1) and value (lanes 32 ..
+      // 32 + D / 4 - 1) first, so that they arrive while the queries are worked on.
+      const bool is_k = lane < 32, kv_valid = lane % 32 < D / 4;
+      const int kv_d0 = kv_valid ? (lane % 32) * 4 : 0;
+      float xn[4] = {0.f, 0.f, 0.f, 0.f};
+      if (has_new) sum_parts4(xn, fin.parts, fin.splits, fin.split_stride, row + (size_t)(is_k ? Hq + kvh : Hq + Hkv + kvh) * D + kv_d0);
       for (int base = 0; base < gd; base += 4 * WAVE) {
         const int e0 = base + lane * 4;
         const bool valid = e0 < gd;
@@ -279,29 +285,24 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
         for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8*>(&qs[wave][r * D + kk * 32 + g * 8]);
       }
       if (has_new) {
-        // The new key (lanes 0 .. D / 4 - 1) and value (lanes 32 .. 32 + D / 4 - 1): into the cache, and
-        // into LDS for this wave's last chunk.
-        const bool is_k = lane < 32, valid = lane % 32 < D / 4;
-        const int d0 = valid ? (lane % 32) * 4 : 0;
-        float x[4];
-        sum_parts4(x, fin.parts, fin.splits, fin.split_stride, row + (size_t)(is_k ? Hq + kvh : Hq + Hkv + kvh) * D + d0);
-        float xk[4] = {x[0], x[1], x[2], x[3]};
-        head_norm_rotate<D>(xk, d0, fin.k_weight, fin.eps, rope_row);
+        // The new key and value: into the cache, and into LDS for this wave's last chunk.
+        float xk[4] = {xn[0], xn[1], xn[2], xn[3]};
+        head_norm_rotate<D>(xk, kv_d0, fin.k_weight, fin.eps, rope_row);
         const int p = kv_len - 1;
         const size_t page = (size_t)table[p / PAGE];
-        if (valid && is_k) {
+        if (kv_valid && is_k) {
           bf16x4 xb;
 #pragma unroll
           for (int e = 0; e < 4; ++e) xb[e] = static_cast<bf16>(xk[e]);
-          *reinterpret_cast<bf16x4*>(&kv_new[d0]) = xb;
-          *reinterpret_cast<bf16x4*>(kc_rw + ((page * Hkv + kvh) * PAGE + p % PAGE) * D + d0) = xb;
+          *reinterpret_cast<bf16x4*>(&kv_new[kv_d0]) = xb;
+          *reinterpret_cast<bf16x4*>(kc_rw + ((page * Hkv + kvh) * PAGE + p % PAGE) * D + kv_d0) = xb;
         }
-        if (valid && !is_k) {
+        if (kv_valid && !is_k) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const bf16 vb = static_cast<bf16>(x[e]);
-            kv_new[D + d0 + e] = vb;
-            vc_rw[((page * Hkv + kvh) * D + d0 + e) * PAGE + p % PAGE] = vb;
+            const bf16 vb = static_cast<bf16>(xn[e]);
+            kv_new[D + kv_d0 + e] = vb;
+            vc_rw[((page * Hkv + kvh) * D + kv_d0 + e) * PAGE + p % PAGE] = vb;
           }
         }
       }
