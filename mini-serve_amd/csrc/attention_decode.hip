@@ -368,29 +368,48 @@ __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __re
   const int b = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const size_t base = ((size_t)b * Hq + head) * splits;
   const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
-  float M = -INFINITY;
-  for (int s0 = 0; s0 < splits; s0 += NB) {
-    float m[NB];
-#pragma unroll
-    for (int u = 0; u < NB; ++u) m[u] = s0 + u < splits ? ml[s0 + u].x : -INFINITY;
-#pragma unroll
-    for (int u = 0; u < NB; ++u) M = fmaxf(M, m[u]);
-  }
-  float L = 0.f, O = 0.f;
-  for (int s0 = 0; s0 < splits; s0 += NB) {
+  float M = -INFINITY, L = 0.f, O = 0.f;
+  if (splits <= NB) {
+    // One round: everything is asked for before the maximum is known.
     float2 q[NB];
     float o[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-      const bool in = s0 + u < splits;
-      q[u] = in ? ml[s0 + u] : make_float2(-INFINITY, 0.f);
-      o[u] = in ? part_o[(base + s0 + u) * D + d] : 0.f;
+      const bool in = u < splits;
+      q[u] = in ? ml[u] : make_float2(-INFINITY, 0.f);
+      o[u] = in ? part_o[(base + u) * D + d] : 0.f;
     }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) M = fmaxf(M, q[u].x);
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
       const float f = q[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(q[u].x - M);  // an empty or absent split adds nothing
       L += q[u].y * f;
       O += o[u] * f;
+    }
+  } else {
+    for (int s0 = 0; s0 < splits; s0 += NB) {
+      float m[NB];
+#pragma unroll
+      for (int u = 0; u < NB; ++u) m[u] = s0 + u < splits ? ml[s0 + u].x : -INFINITY;
+#pragma unroll
+      for (int u = 0; u < NB; ++u) M = fmaxf(M, m[u]);
+    }
+    for (int s0 = 0; s0 < splits; s0 += NB) {
+      float2 q[NB];
+      float o[NB];
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const bool in = s0 + u < splits;
+        q[u] = in ? ml[s0 + u] : make_float2(-INFINITY, 0.f);
+        o[u] = in ? part_o[(base + s0 + u) * D + d] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const float f = q[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(q[u].x - M);
+        L += q[u].y * f;
+        O += o[u] * f;
+      }
     }
   }
   const int tok = tokens ? tokens[b] : b;
