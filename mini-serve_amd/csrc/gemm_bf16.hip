@@ -569,6 +569,28 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
   return launch_status();
 }
 
+// Width of the 128-row tiles of a product: 64, 128 or 192 columns. All blocks of up to 512 (two per CU)
+// run at once, so what counts is how many such rounds the tiles make and how long a tile of each width
+// takes (measured at 2,048 rows, relative to 128 columns): a 192-wide tile does 1.5 times the work in
+// 1.4 times the time, a 64-wide one half the work in 0.62; a few rounds count whole, many as they are.
+static int wide_tile_cols(int M, int N, int splits) {
+  const int widths[3] = {128, 192, 64};
+  const double tile_time[3] = {1.0, 1.4, 0.62};
+  const long row_tiles = (M + 127) / 128;
+  int best = 128;
+  double least = 0;
+  for (int i = 0; i < 3; ++i) {
+    const long tiles = row_tiles * ((N + widths[i] - 1) / widths[i]) * splits;
+    const double rounds = tiles <= 1024 ? (double)((tiles + 511) / 512) : tiles / 512.0;
+    const double t = rounds * tile_time[i];
+    if (i == 0 || t < least * 0.97) {  // another width has to be clearly better
+      least = t;
+      best = widths[i];
+    }
+  }
+  return best;
+}
+
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
 // its loads at once, unless that would make more waves than the chip holds a few times over (then
 // slices of several whole slabs). With up to 16 rows the partial sums are small beside the weights
@@ -729,7 +751,12 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
   }
   if (M <= 64 || K % BK) return MS_UNSUPPORTED;
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (big >= 256) return launch_dma<128, 128, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  if (big >= 256) {
+    const int cols = wide_tile_cols(M, N, 1);
+    if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+    if (cols == 64) return launch_dma<128, 64, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+    return launch_dma<128, 128, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  }
   if ((long)((M + 63) / 64) * ((N + 63) / 64) >= 256) return launch_dma<64, 64, BK, 2, 4>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
   return MS_UNSUPPORTED;  // too few tiles without a split of K
 }
@@ -764,7 +791,12 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
   // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
   if (K % BK == 0 && ldx % 8 == 0) {
-    if (big >= 256) return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    if (big >= 256) {
+      const int cols = wide_tile_cols(M, N, splits);
+      if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+      if (cols == 64) return launch_dma<128, 64, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+      return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    }
     return launch_dma<64, 64, BK, 2, 4>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
   }
   if (big >= 256) {

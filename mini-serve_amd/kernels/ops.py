@@ -79,8 +79,28 @@ def library_path() -> str:
     return str(build.build_kernels())
 
 
+_pinned_stream: int | None = None
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _pinned_stream if _pinned_stream is not None else torch.cuda.current_stream().cuda_stream
+
+
+class stream_scope:
+    """Looks the current HIP stream up once for all kernel launches inside the ``with`` block (the
+    lookup costs several microseconds, a model pass makes hundreds). The stream must not be switched
+    inside the block."""
+
+    def __enter__(self):
+        global _pinned_stream
+        self._before = _pinned_stream
+        _pinned_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self._before
+        return False
 
 
 def _check(code: int, what: str) -> None:

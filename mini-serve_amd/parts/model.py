@@ -94,6 +94,10 @@ class DecoderModel:
     def forward(self, batch, pool):
         """Run the batch's tokens through every run-order entry and return float32 logits
         ``[len(batch.want_rows), vocab]`` at the wanted flat token indices."""
+        with self.rt.ops.stream_scope():
+            return self._forward(batch, pool)
+
+    def _forward(self, batch, pool):
         batch.memo = {}  # what parts share between layers is made anew in every pass (a captured pass records it)
         residual = self.embedding.forward(batch.token_ids)
         pending = None  # a sum a layer left to be added to the residual stream by its next reader
