@@ -34,7 +34,8 @@ struct DecodeTile {
 
 // The fused form takes, instead of finished queries and a cache that already holds the new token, the
 // qkv projection as it leaves the small-M product: float partial sums [splits, tokens, (Hq + 2 Hkv) D].
-// Every wave sums, norms and rotates the queries of its KV head's group itself (a few hundred floats);
+// Every wave sums, norms and rotates the queries of its KV head's group itself (up to 256 floats; the
+// block's waves share the work if there are more);
 // the one wave whose chunks end with the sequence's last token does the same for the new key, takes
 // the new value, stores both into the cache and puts them into its operands of that chunk in
 // registers (what its loads brought from the not yet written slot is replaced, so no store has to be
@@ -266,8 +267,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
       const int kv_d0 = kv_valid ? (lane % 32) * 4 : 0;
       float xn[4] = {0.f, 0.f, 0.f, 0.f};
       if (has_new) sum_parts4(xn, fin.parts, fin.splits, fin.split_stride, row + (size_t)(is_k ? Hq + kvh : Hq + Hkv + kvh) * D + kv_d0);
-      for (int base = 0; base < gd; base += 4 * WAVE) {
-        const int e0 = base + lane * 4;
+      // Up to 256 floats (a lane's four of one round): every wave works its own copy out, no barrier.
+      // More: the block's waves share the work (a wave takes whole heads) and meet once.
+      const bool together = gd > 4 * WAVE;
+      const int step = together ? 4 * 256 : 4 * WAVE;
+      bf16* q_lds = together ? &qs[0][0] : &qs[wave][0];
+      for (int base = 0; base < gd; base += step) {
+        const int e0 = base + (together ? tid : lane) * 4;
         const bool valid = e0 < gd;
         const int ec = valid ? e0 : 0;
         float x[4];
@@ -277,12 +283,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
           bf16x4 xb;
 #pragma unroll
           for (int e = 0; e < 4; ++e) xb[e] = static_cast<bf16>(x[e]);
-          *reinterpret_cast<bf16x4*>(&qs[wave][ec]) = xb;
+          *reinterpret_cast<bf16x4*>(q_lds + ec) = xb;
         }
       }
+      if (together) __syncthreads();
       if (r < G) {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8*>(&qs[wave][r * D + kk * 32 + g * 8]);
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8*>(q_lds + r * D + kk * 32 + g * 8);
       }
       if (has_new) {
         // The new key and value: into the cache, and into LDS for this wave's last chunk.
