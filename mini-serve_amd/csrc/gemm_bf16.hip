@@ -492,6 +492,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_small_kernel(const bf16* __rest
   }
   // acc[i][e] = C[m = 16 i + r][n = nb + 4 g + e]
   float* dst = P + (size_t)split * M * N;
+  if (SHARED && MB == 1 && N % 4 == 0) {
+    // A wave's own store would put 64 bytes into each of up to 16 rows: half cache lines, which the
+    // memory system takes at a fraction of its rate (at 8 rows the partial sums of a 24576 x 4096
+    // matrix cost as much as 15 % of its weights). The block's four waves meet in LDS instead and
+    // write their 64 columns of a row as one run of 256 bytes.
+    float* outs = reinterpret_cast<float*>(xs);  // 16 rows x 64 columns
+    static_assert(!SHARED || MB * 16 * XS_STRIDE * 2 >= 16 * 64 * 4, "the X slab's memory holds the block's results");
+    __syncthreads();  // every wave is done with the last slab
+    *reinterpret_cast<floatx4*>(&outs[r * 64 + wave * 16 + g * 4]) = acc[0];
+    __syncthreads();
+    const int m = tid / 16, n = row_block * 64 + (tid % 16) * 4;
+    if (m < M && n < N) *reinterpret_cast<floatx4*>(dst + (size_t)m * N + n) = *reinterpret_cast<const floatx4*>(&outs[m * 64 + (tid % 16) * 4]);
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < MB; ++i) store4(dst, 1, i * 16 + r, nb + g * 4, M, N, N, acc[i], N % 4 == 0);
 }
