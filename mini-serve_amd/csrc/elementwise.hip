@@ -24,6 +24,26 @@ extern "C" int ms_embed(const int* ids, const void* table, int table_is_bf16, fl
 }
 
 // ---------------------------------------------------------------------------------------------
+// Token ids that are still on the device: the last token of row i becomes src[feed[i]] where
+// feed[i] >= 0 (a token an earlier step sampled and the host has not read back yet). row_start holds
+// rows + 1 offsets into ids; nullptr: every row is one token.
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ row_start, const int* __restrict__ feed,
+                                   const int* __restrict__ src, int rows, int src_len) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows) return;
+  const int f = feed[i];
+  if (f < 0 || f >= src_len) return;
+  ids[row_start ? row_start[i + 1] - 1 : i] = src[f];
+}
+
+extern "C" int ms_feed_tokens(int* ids, const int* row_start, const int* feed, const int* src, int rows, int src_len, hipStream_t st) {
+  if (rows <= 0) return MS_OK;
+  if (ids == nullptr || feed == nullptr || src == nullptr || src_len <= 0) return MS_BAD_ARG;
+  feed_tokens_kernel<<<(rows + 255) / 256, 256, 0, st>>>(ids, row_start, feed, src, rows, src_len);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
 // y[r, :] = w * x[row(r), :] * rsqrt(mean(x^2) + eps), float32 throughout, rounded once.
 // With `parts` (float [splits, rows_total, width], the partial sums of a matrix product that still
 // has to be added to the residual stream) the row is first brought up to date: x[row] + sum over

@@ -23,6 +23,9 @@ class StepRow:
     cache: object  # RequestCache
     tokens: list
     want: list  # indices into ``tokens`` whose logits are asked for
+    # The row's last token is not known on the host yet: it is element ``feed`` of the device tensor
+    # of sampled tokens that the step is given (``tokens[-1]`` is ignored). None: all tokens are known.
+    feed: int | None = None
 
 
 @dataclass
@@ -39,7 +42,7 @@ class StepBatch:
     __slots__ = (
         "num_rows", "num_tokens", "num_wanted", "token_ids", "positions", "token_row", "row_start", "starts",
         "kv_lens", "state_slots", "want_rows", "groups", "row_lens", "row_starts_host", "max_kv_len", "is_decode",
-        "num_decode_tokens", "decode_tokens", "prefill_tokens", "_tiles", "memo",
+        "num_decode_tokens", "decode_tokens", "prefill_tokens", "_tiles", "memo", "feed",
     )
 
     def __init__(self):
@@ -103,6 +106,9 @@ class BatchBuilder:
         take("ids", T); take("pos", T); take("row", T)
         take("row_start", B + 1); take("starts", B); take("kv_lens", B); take("state", B)
         take("want", n_want)
+        fed = any(r.feed is not None for r in rows)
+        if fed:
+            take("feed", B)
         n_dec = sum(1 for n in lens if n == 1)
         mixed = 0 < n_dec < B
         if mixed:
@@ -144,6 +150,8 @@ class BatchBuilder:
                     pre[q : q + n] = np.arange(t, t + n, dtype=np.int32)
                     q += n
                 t += n
+        if fed:
+            view("feed")[:] = [-1 if r.feed is None else r.feed for r in rows]
         view("starts")[:] = starts
         view("kv_lens")[:] = [s + n for s, n in zip(starts, lens)]
         view("state")[:] = [r.cache.state_slot if r.cache.state_slot is not None else 0 for r in rows]
@@ -169,6 +177,7 @@ class BatchBuilder:
         b.token_ids, b.positions, b.token_row = dview("ids"), dview("pos"), dview("row")
         b.row_start, b.starts, b.kv_lens, b.state_slots = dview("row_start"), dview("starts"), dview("kv_lens"), dview("state")
         b.want_rows = dview("want")
+        b.feed = dview("feed") if fed else None
         b.groups = [GroupBatch(dview(f"table{g}").view(B, widths[g]), dview(f"slots{g}")) for g in range(self.num_groups)]
         b.row_lens = lens
         b.row_starts_host = list(starts)

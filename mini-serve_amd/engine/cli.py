@@ -39,7 +39,7 @@ def add_engine_args(parser: argparse.ArgumentParser) -> None:
     g.add_argument("--disable-radix", action="store_true",
                    help="no prefix cache" + _NO_EFFECT + "prefixes are never shared between requests)")
     g.add_argument("--disable-overlap", action="store_true",
-                   help="read back each step's tokens before scheduling the next" + _NO_EFFECT + "steps are always synchronous)")
+                   help="read back each step's tokens before scheduling the next (default: one step later)")
     g.add_argument("--attn-workspace-mb", type=int, default=None,
                    help="attention scratch buffer in MiB" + _NO_EFFECT + "the attention kernels size their own scratch)")
     g.add_argument("--fused-ops", action="store_true",
@@ -59,4 +59,5 @@ def engine_kwargs(args: argparse.Namespace) -> dict:
         block_backend=args.block_backend,
         page_size=args.page_size,
         kv_mem_fraction=args.kv_mem_fraction,
+        overlap=not args.disable_overlap,
     )

@@ -1,12 +1,19 @@
-"""The engine loop: ``step()`` = schedule -> one step of the model -> sample -> read back -> retire.
+"""The engine loop: ``step()`` = schedule -> one step of the model -> sample -> read back -> retire,
+with the read-back lagging one step behind by default.
 
 Interface in the reference's manner (miniserve/engine/engine.py:41-211): ``Engine(model, **options)``,
 ``add_request(prompt_ids, SamplingParams) -> Request``, ``step() -> Batch | None``, ``abort(rid)``,
 ``generate(prompts, params) -> list[list[int]]``, ``has_unfinished``, ``logits_hook``. Token ids in,
 token ids out; the engine never tokenizes.
 
-Each step is synchronous: the sampled tokens are read back (one copy of ``[rows]`` int32) before the
-next step is scheduled. Only the rows that complete their sequence in a step ask for logits and are
+Overlap (one-step lag, miniserve/engine/engine.py:9-21,137-147,167-198): step t + 1 is scheduled and
+launched before the tokens of step t are read back, so the device never waits for the host's
+bookkeeping. Until then a sampled token stands in its request's output as ``PLACEHOLDER``; the next
+step takes it from the device tensor the sampler left (``StepRow.feed``). What the host learns one
+step late is a stop token: the request has then run one step too many, and the token that step
+sampled for it is dropped. Stops by length are known in advance and cost nothing. With
+``overlap=False`` every step's tokens are read back (one copy of ``[rows]`` int32) before the next
+step is scheduled. Only the rows that complete their sequence in a step ask for logits and are
 sampled; a portion of a prompt that stops short asks for none (the reference computes and discards
 a row for it, miniserve/engine/engine.py:156-172).
 """
@@ -16,11 +23,26 @@ from __future__ import annotations
 import itertools
 import random
 from collections.abc import Sequence
+from dataclasses import dataclass
+
+import torch
 
 from .batch import StepRow
 from .policy import make_policy
-from .request import Request, RequestState, SamplingParams
+from .request import PLACEHOLDER, Request, RequestState, SamplingParams
 from .scheduler import Batch, Scheduler
+
+
+@dataclass
+class _Launched:
+    """A step that has been handed to the device (miniserve/engine/engine.py:214-221)."""
+
+    batch: Batch
+    sampling: list  # the requests that sample a token in this step, in row order
+    places: list  # per such request: the index in its output where the token goes
+    tokens: object = None  # int32 [len(sampling)] where the sampler left them
+    host: object = None  # the same on the host once ``ready`` has passed
+    ready: object = None  # event after the copy to the host (None: ``host`` is valid already)
 
 DEFAULT_CHUNKED_PREFILL = 2048
 
@@ -42,6 +64,7 @@ class Engine:
         decode_graph_max_bs: int | None = None,
         block_backend: str | None = None,
         sampler=None,
+        overlap: bool = True,
     ):
         """``kv_pool_tokens``: exact cache pool size in tokens (default: as large as memory allows).
         ``chunked_prefill_size``: token budget per step with prompts cut into portions and batched
@@ -50,7 +73,8 @@ class Engine:
         ``decode_graph_max_bs`` requests (default ``max_running``).
         ``block_backend``: ``python`` or ``cpp`` page bookkeeping.
         ``seed``: seeds the sampling of requests submitted without a seed of their own, in
-        submission order. ``runner``: use this model runner instead of building one for ``model``."""
+        submission order. ``runner``: use this model runner instead of building one for ``model``.
+        ``overlap``: launch the next step before the tokens of this one are read back."""
         if chunked_prefill_size is None:
             chunked_prefill_size = DEFAULT_CHUNKED_PREFILL
         if runner is None:
@@ -84,6 +108,9 @@ class Engine:
         self.logits_hook = None  # called with (batch, logits of the completing rows) before sampling
         self.launched: Batch | None = None
         self.num_steps = 0
+        self.overlap = overlap
+        self._inflight: _Launched | None = None  # launched, tokens not read back yet
+        self.dropped_tokens = 0  # sampled for a request that had already ended (overlap only)
 
     # ------------------------------------------------------------------ requests
 
@@ -108,33 +135,68 @@ class Engine:
     # ------------------------------------------------------------------ the loop
 
     def step(self) -> Batch | None:
-        """Run one step; returns the batch it ran (its requests now carry their new tokens), or None
-        when idle."""
+        """Schedule and launch one step; read back, and return the batch of, the step whose tokens
+        are due: this one without overlap, the previous one with it (None when there is none)."""
+        prev, self._inflight = self._inflight, None
         batch = self.scheduler.schedule()
         self.launched = batch
-        if batch is None:
-            return None
+        launched = self._launch(batch, prev) if batch is not None else None
+        if not self.overlap:
+            return self._finish(launched) if launched is not None else None
+        self._inflight = launched
+        return self._finish(prev) if prev is not None else None
+
+    def _launch(self, batch: Batch, prev: _Launched | None) -> _Launched:
         completes = batch.completes()
-        rows = [
-            StepRow(r.cache, r.token_slice(s, n), [n - 1] if done else [])
-            for r, s, n, done in zip(batch.requests, batch.starts, batch.extend_lens, completes)
-        ]
-        logits = self.runner.step(rows)
+        source = {id(r): i for i, r in enumerate(prev.sampling)} if prev is not None else {}
+        rows = []
+        for r, s, n, done in zip(batch.requests, batch.starts, batch.extend_lens, completes):
+            tokens = r.token_slice(s, n)
+            # Only a request's last token can be outstanding, and only from the step before this one.
+            feed = source[id(r)] if tokens[-1] == PLACEHOLDER else None
+            rows.append(StepRow(r.cache, tokens, [n - 1] if done else [], feed))
+        if any(row.feed is not None for row in rows):
+            logits = self.runner.step(rows, feed_from=prev.tokens)
+        else:
+            logits = self.runner.step(rows)
         self.num_steps += 1
         sampling = [r for r, done in zip(batch.requests, completes) if done]
+        launched = _Launched(batch, sampling, [len(r.output_ids) for r in sampling])
         if not sampling:
-            return batch
+            return launched
         if self.logits_hook is not None:
             self.logits_hook(batch, logits)
-        tokens = self.sampler.sample(logits, self.sampler.prepare(sampling)).tolist()
-        for r, tok in zip(sampling, tokens):
-            r.output_ids.append(tok)
+        launched.tokens = self.sampler.sample(logits, self.sampler.prepare(sampling))
+        if launched.tokens.is_cuda:
+            launched.host = torch.empty(launched.tokens.shape, dtype=launched.tokens.dtype, pin_memory=True)
+            launched.host.copy_(launched.tokens, non_blocking=True)
+            launched.ready = torch.cuda.Event()
+            launched.ready.record()
+        else:
+            launched.host = launched.tokens
+        for r in sampling:
+            r.output_ids.append(PLACEHOLDER)
             if r.state is RequestState.PREFILL:
                 r.transition(RequestState.DECODE)
-            if r.should_stop():
+        return launched
+
+    def _finish(self, launched: _Launched) -> Batch:
+        """Read the step's tokens back, put them in their places, end what they end."""
+        if not launched.sampling:
+            return launched.batch
+        if launched.ready is not None:
+            launched.ready.synchronize()
+        for r, at, tok in zip(launched.sampling, launched.places, launched.host.tolist()):
+            if r.is_done:  # aborted, or ended by the token before this one
+                self.dropped_tokens += 1
+                continue
+            r.output_ids[at] = tok
+            if at + 1 >= r.params.max_new_tokens or tok in r.params.stop_token_ids:
+                self.dropped_tokens += len(r.output_ids) - (at + 1)
+                del r.output_ids[at + 1 :]  # a placeholder of the step already under way
                 r.transition(RequestState.FINISHED)
                 self._retire(r)
-        return batch
+        return launched.batch
 
     def _retire(self, req: Request) -> None:
         if req.cache is not None:

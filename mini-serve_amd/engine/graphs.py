@@ -61,7 +61,7 @@ class DecodeGraphs:
     def _layout(self, g: int, w: int):
         seg, off = {}, 0
         for name, n in [("ids", g), ("pos", g), ("row", g), ("row_start", g + 1), ("starts", g), ("kv_lens", g),
-                        ("state", g), ("want", g)] + [
+                        ("state", g), ("want", g), ("feed", g)] + [
             item for k in range(self.num_groups) for item in ((f"slots{k}", g), (f"table{k}", g * w))
         ]:
             seg[name] = (off, n)
@@ -94,6 +94,7 @@ class DecodeGraphs:
         b.token_ids, b.positions, b.token_row = dv("ids"), dv("pos"), dv("row")
         b.row_start, b.starts, b.kv_lens, b.state_slots = dv("row_start"), dv("starts"), dv("kv_lens"), dv("state")
         b.want_rows = dv("want")
+        b.feed = None  # tokens still on the device are put into the static buffer before the replay
         b.groups = [GroupBatch(dv(f"table{k}").view(g, w), dv(f"slots{k}")) for k in range(self.num_groups)]
         b.row_lens, b.row_starts_host, b.max_kv_len, b.is_decode = [1] * g, [0] * g, w * self.runner.page_size, True
         b.num_decode_tokens, b.decode_tokens, b.prefill_tokens = g, None, None
@@ -134,8 +135,9 @@ class DecodeGraphs:
             o, _ = c.seg[f"table{k}"]
             h[o + first * w : o + g * w] = dummy
 
-    def run(self, rows, starts):
-        """Replay the graph for these decode rows (their tables already hold the new token)."""
+    def run(self, rows, starts, feed_from=None):
+        """Replay the graph for these decode rows (their tables already hold the new token). Rows with
+        ``feed`` take their token from the device tensor ``feed_from``."""
         from ..cache.table import pack_tables
 
         g, w = key = self._key(rows)
@@ -151,6 +153,10 @@ class DecodeGraphs:
             return h[o : o + n]
 
         hv("ids")[:B] = [r.tokens[0] for r in rows]
+        fed = any(r.feed is not None for r in rows)
+        if fed:
+            hv("feed")[:B] = [-1 if r.feed is None else r.feed for r in rows]
+            hv("feed")[B:] = -1
         hv("pos")[:B] = starts
         hv("starts")[:B] = starts
         hv("kv_lens")[:B] = [s + 1 for s in starts]
@@ -165,5 +171,8 @@ class DecodeGraphs:
             self._fill_padding(c, B, g, w)
         c.dev.copy_(c.host, non_blocking=True)
         c.fence.record()
+        if fed:
+            o, n = c.seg["feed"]
+            self.runner.model.rt.ops.feed_tokens(c.batch.token_ids, None, c.dev[o : o + n], feed_from)
         c.graph.replay()
         return c.logits[:B]

@@ -90,10 +90,12 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ the step function
 
-    def step(self, rows: list[StepRow]) -> torch.Tensor | None:
+    def step(self, rows: list[StepRow], feed_from: torch.Tensor | None = None) -> torch.Tensor | None:
         """Run one batch. Each row's tokens continue its cache at position ``cache.num_tokens``.
         Returns float32 logits ``[sum(len(row.want)), vocab]`` in row order (None if nothing is
-        wanted). Raises ``OutOfBlocks`` with every table unchanged if the pool cannot hold the step."""
+        wanted). Raises ``OutOfBlocks`` with every table unchanged if the pool cannot hold the step.
+        ``feed_from``: int32 device tensor of tokens an earlier step sampled; a row with ``feed = i``
+        runs ``feed_from[i]`` as its last token (the host need not have read it back)."""
         if not rows:
             return None
         vocab = self.model.vocab_size
@@ -104,8 +106,13 @@ class ModelRunner:
             seen.add(id(r.cache))
             if not r.tokens:
                 raise ValueError("a row without tokens")
-            if min(r.tokens) < 0 or max(r.tokens) >= vocab:
+            known = r.tokens if r.feed is None else r.tokens[:-1]
+            if known and (min(known) < 0 or max(known) >= vocab):
                 raise ValueError(f"token id out of range [0, {vocab})")
+            if r.feed is not None:
+                if feed_from is None or not 0 <= r.feed < feed_from.shape[0]:
+                    raise ValueError("a row is fed from the device but no such token was given")
+                r.tokens = known + [0]
             if r.want and not (0 <= min(r.want) and max(r.want) < len(r.tokens)):
                 raise ValueError("wanted place outside the row's tokens")
         need = [0] * self.cache.num_groups
@@ -119,10 +126,12 @@ class ModelRunner:
         for r in rows:
             self.cache.extend(r.cache, len(r.tokens))
         if self.graphs is not None and self.graphs.usable(rows):
-            logits = self.graphs.run(rows, starts)
+            logits = self.graphs.run(rows, starts, feed_from)
             self.graph_steps += 1
         else:
             batch = self.builder.build(rows, starts)
+            if batch.feed is not None:
+                self.model.rt.ops.feed_tokens(batch.token_ids, batch.row_start, batch.feed, feed_from)
             logits = self.model.forward(batch, self.pool)
         for r in rows:
             self.cache.advance(r.cache)

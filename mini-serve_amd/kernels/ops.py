@@ -22,6 +22,7 @@ _ERRORS = {1: "bad argument", 2: "unsupported size", 3: "kernel launch failed"}
 
 _SIGNATURES = {
     "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
+    "ms_feed_tokens": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int, _c_ll, _c_void],
     "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -165,6 +166,24 @@ def embed(token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     _check(library().ms_embed(token_ids.data_ptr(), table.data_ptr(), int(table.dtype == BF16), out.data_ptr(),
                               token_ids.shape[0], table.shape[1], _stream()), "embed")
     return out
+
+
+def feed_tokens(token_ids: torch.Tensor, row_start: torch.Tensor | None, feed: torch.Tensor, source: torch.Tensor) -> None:
+    """In place: the last token of row ``i`` of ``token_ids`` becomes ``source[feed[i]]`` where
+    ``feed[i] >= 0``. ``row_start``: ``rows + 1`` offsets of the rows in ``token_ids`` (None: one token
+    per row). For tokens that were sampled on the device and not yet read back."""
+    _dev(token_ids, "token_ids", I32, 1)
+    _dev(feed, "feed", I32, 1)
+    _dev(source, "source", I32, 1)
+    rows = feed.shape[0]
+    if row_start is not None:
+        _dev(row_start, "row_start", I32, 1)
+        if row_start.shape[0] != rows + 1:
+            raise ValueError("row_start must hold one offset more than there are rows")
+    elif token_ids.shape[0] < rows:
+        raise ValueError("fewer tokens than rows")
+    _check(library().ms_feed_tokens(token_ids.data_ptr(), _ptr(row_start), feed.data_ptr(), source.data_ptr(), rows,
+                                    source.shape[0], _stream()), "feed_tokens")
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None,

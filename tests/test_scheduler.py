@@ -8,7 +8,7 @@ import random
 import pytest
 
 from miniserve_amd.engine.engine import Engine
-from miniserve_amd.engine.request import InvalidTransition, Request, RequestState, SamplingParams
+from miniserve_amd.engine.request import PLACEHOLDER, InvalidTransition, Request, RequestState, SamplingParams
 from miniserve_amd.engine.scheduler import Phase, Scheduler
 from toy_runner import ToyRunner, ToySampler, run_alone
 
@@ -275,26 +275,30 @@ def test_windowed_groups_let_more_requests_in():
 # ------------------------------------------------------------------------------------------ the loop under load
 
 
-def toy_engine(pages, chunk, windows=(0,), max_running=8, backend="python", seed=0):
+def toy_engine(pages, chunk, windows=(0,), max_running=8, backend="python", seed=0, overlap=True):
     runner = ToyRunner(pages, page_size=4, windows=windows, max_running=max_running, max_step_tokens=chunk or None, backend=backend)
     return Engine(None, max_running=max_running, max_prefill_tokens=64, runner=runner, chunked_prefill_size=chunk,
-                  seed=seed, sampler=ToySampler())
+                  seed=seed, sampler=ToySampler(), overlap=overlap)
 
 
+@pytest.mark.parametrize("overlap", [True, False])
 @pytest.mark.parametrize("pages,chunk,windows,backend", [
     (8, 3, (0,), "python"), (16, 0, (0,), "cpp"), (64, 2048, (0,), "python"), (8, 5, (0, 6), "cpp"), (12, 7, (10,), "python"),
 ])
-def test_load_under_page_pressure(pages, chunk, windows, backend):
+def test_load_under_page_pressure(pages, chunk, windows, backend, overlap):
+    """As the reference's load test (tests/test_engine.py:562-598): random requests and arrivals, pools
+    that force preemption, whole and chunked prefill, the read-back one step behind or not; every
+    output equals the request's run alone."""
     preemptions = 0
     for seed in range(6):
-        preemptions += _load(seed, pages, chunk, windows, backend)
+        preemptions += _load(seed, pages, chunk, windows, backend, overlap)
     if pages == 8:
         assert preemptions > 0, "the small pool was meant to force preemption"
 
 
-def _load(seed, pages, chunk, windows, backend) -> int:
+def _load(seed, pages, chunk, windows, backend, overlap=True) -> int:
     rng = random.Random(seed)
-    eng = toy_engine(pages, chunk, windows, backend=backend, seed=seed)
+    eng = toy_engine(pages, chunk, windows, backend=backend, seed=seed, overlap=overlap)
     vocab = eng.runner.model.vocab_size
     submitted = []
     pending = []
@@ -333,9 +337,68 @@ def test_engine_assigns_seeds_in_submission_order():
     assert a.add_request([1], SamplingParams(1, seed=77)).seed == 77
 
 
-def test_abort_at_any_time_returns_everything():
+def test_overlap_drops_what_runs_past_a_stop():
+    """With the read-back one step behind, a request that samples its stop token has already been
+    launched once more: that token is dropped and the outputs are what the synchronous loop gives.
+    (The reference counts the same cases, tests/test_engine.py:601-641.)"""
+    dropped = 0
+    for seed in range(12):
+        outs = []
+        for overlap in (True, False):
+            rng = random.Random(seed)
+            eng = toy_engine(8, 3, seed=seed, overlap=overlap)
+            vocab = eng.runner.model.vocab_size
+            reqs = [eng.add_request([rng.randrange(vocab) for _ in range(rng.randint(1, 9))],
+                                    SamplingParams(rng.randint(1, 14), temperature=4.0, seed=rng.randrange(2**32),
+                                                   stop_token_ids=frozenset(rng.sample(range(vocab), 8))))
+                    for _ in range(12)]
+            steps = 0
+            while eng.has_unfinished:
+                eng.step()
+                eng.runner.cache.check_invariants()
+                steps += 1
+                assert steps < 3000
+            assert eng.runner.cache.idle and all(PLACEHOLDER not in r.output_ids for r in reqs)
+            outs.append([r.output_ids for r in reqs])
+            if overlap:
+                dropped += eng.dropped_tokens
+            else:
+                assert eng.dropped_tokens == 0
+        assert outs[0] == outs[1]
+    assert dropped > 0, "no request ran past its stop token: the case was meant to occur"
+
+
+def test_overlap_request_ends_while_it_waits_after_a_preemption(monkeypatch):
+    """Two requests of 7 tokens in a pool of 4 pages of 4: both decode until each needs a third page, and
+    the newer one is preempted, while the token of its last step is still on its way. That token is its
+    stop token: it ends from WAITING, and never runs again."""
+    seen = []
+    plain_transition = Request.transition
+
+    def recording(self, new):
+        seen.append((self.rid, self.state, new))
+        plain_transition(self, new)
+
+    monkeypatch.setattr(Request, "transition", recording)
+    vocab, prompt_a, prompt_b = 50, [3, 1, 4, 1, 5, 9, 2], [2, 7, 1, 8, 2, 8, 1]
+    alone = run_alone(prompt_b, SamplingParams(9), 5, vocab)
+    assert alone[0] != alone[1], "the second token was meant to be the first stop"
+    eng = toy_engine(4, 16, seed=0, overlap=True)
+    a = eng.add_request(prompt_a, SamplingParams(9, seed=4))
+    b = eng.add_request(prompt_b, SamplingParams(9, seed=5, stop_token_ids=frozenset({alone[1]})))
+    while eng.has_unfinished:
+        eng.step()
+        eng.runner.cache.check_invariants()
+    assert b.output_ids == alone[:2] and a.output_ids == run_alone(prompt_a, a.params, 4, vocab)
+    assert (b.rid, RequestState.DECODE, RequestState.WAITING) in seen, "the newer request was meant to be preempted"
+    assert (b.rid, RequestState.WAITING, RequestState.FINISHED) in seen
+    assert eng.scheduler.num_preemptions == 1 and eng.runner.cache.idle
+
+
+@pytest.mark.parametrize("overlap", [True, False])
+def test_abort_at_any_time_returns_everything(overlap):
     for at in range(0, 12, 2):
-        eng = toy_engine(16, 4)
+        eng = toy_engine(16, 4, overlap=overlap)
         rs = [eng.add_request(list(range(1, 10)), SamplingParams(10)) for _ in range(3)]
         for _ in range(at):
             eng.step()

@@ -50,7 +50,11 @@ class ToyRunner:
         self.history.pop(id(rc), None)
         self.cache.release(rc)
 
-    def step(self, rows):
+    def step(self, rows, feed_from=None):
+        for r in rows:  # a token that is "still on the device": the last of the row
+            if getattr(r, "feed", None) is not None:
+                r.tokens = list(r.tokens[:-1]) + [int(feed_from[r.feed])]
+        assert all(t >= 0 for r in rows for t in r.tokens), "a placeholder reached the model"
         need = [0] * self.cache.num_groups
         for r in rows:
             for g, k in enumerate(self.cache.pages_needed(r.cache, len(r.tokens))):
