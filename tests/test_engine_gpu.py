@@ -88,6 +88,39 @@ def test_stop_token_is_kept(folders):
     assert eng.generate([prompt], SamplingParams(max_new_tokens=10, stop_token_ids=frozenset({stop}))) == [cut]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graph", [True, False])
+def test_read_back_one_step_behind_changes_nothing(folders, dtype, graph):
+    """The engine launches a step before it has read the previous one's tokens (they reach the next
+    step on the device, through the uploaded ids or a captured graph's static buffer): same outputs
+    as with a read-back after every step, with stop tokens that end requests one step late, sampled
+    requests, and a pool that forces preemption."""
+    from miniserve_amd.engine.request import PLACEHOLDER, SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyB"])
+    prompts = prompts_for(cfg, [30, 45, 20, 38, 25, 41, 3, 17], seed=9)
+    plain = {i: P.greedy(cfg, w, prompts[i], 6) for i in (2, 4)} if dtype == "float32" else {}  # greedy, no stops
+    outs = {}
+    for overlap in (True, False):
+        eng = engine(folders["tinyB"], dtype, kv_pool_tokens=16 * 14, max_running=6, chunked_prefill_size=32,
+                     decode_graph=graph, overlap=overlap)
+        reqs = []
+        for i, p in enumerate(prompts):
+            stops = frozenset(range(0, cfg["vocab_size"], 9)) if i % 2 else frozenset()  # every ninth token ends odd requests
+            reqs.append(eng.add_request(p, SamplingParams(20 + i, stop_token_ids=stops, temperature=0.0 if i % 3 else 0.9, seed=i)))
+        while eng.has_unfinished:
+            eng.step()
+        assert eng.runner.cache.idle and all(PLACEHOLDER not in r.output_ids for r in reqs)
+        assert eng.scheduler.num_preemptions > 0, "the pool was meant to be too small"
+        outs[overlap] = [r.output_ids for r in reqs]
+        if overlap:
+            assert eng.dropped_tokens > 0, "no request ran past a stop token"
+            assert not graph or eng.runner.graph_steps > 0
+    assert outs[True] == outs[False]
+    for i, want in plain.items():
+        assert outs[True][i][:6] == want
+
+
 def test_sampled_requests_reproduce_beside_greedy_ones(folders):
     """Temperature sampling with a request seed: the same tokens alone, in a batch, and after
     preemption; equal to the plain sampler run on the plain logits."""
