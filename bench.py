@@ -4,7 +4,8 @@ bfloat16, batch 8 at a context of 4,096 tokens per request, 16-token pages.
     python bench.py --gpus 1 --steps K --warmup W
 
 A "step" is one decode step of the engine (schedule, one pass of the model over the batch's last
-tokens, sampling on the device, one read-back of the tokens). Requests are prefilled through the
+tokens, sampling on the device, one read-back of the tokens, which the engine waits for one step
+after the launch). Requests are prefilled through the
 same step function in portions of 2,048 tokens; the timed steps are the last K before every
 request reaches the context length. One JSON line is printed, with ``value`` = decoded tokens per
 second, plus the prefill rate of one 2,048-token prompt, the decode step's share of the HBM
@@ -124,7 +125,7 @@ def main() -> int:
             "parallelism": "single GPU", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
-            "page_size": 16, "decode_graph": not args.no_graph,
+            "page_size": 16, "decode_graph": not args.no_graph, "overlap": True,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
