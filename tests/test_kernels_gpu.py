@@ -167,13 +167,15 @@ def test_gemm_bf16(ops, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024),
-                                   (4000, 1500, 192), (1990, 1000, 128)])
+                                   (4000, 1500, 192), (1990, 1000, 128), (2048, 6100, 128), (2048, 1000, 256)])
 def test_gemm_bf16_large_tiles(ops, m, n, k):
     """Shapes with at least 256 tiles of 128 x 128 and K a multiple of 64 take the kernel whose slabs go
     straight into LDS: edge tiles in both directions (rows past the end are read from the last valid
     row and never stored), one slab, an odd number of slabs. The last two have many more rows than
     columns and tile counts that divide by the XCD grid (2 x 4 with 128-wide tiles, 4 x 2 with 64-wide
-    ones): each XCD then owns a rectangle of tiles, with the matrix's edges in some of them."""
+    ones): each XCD then owns a rectangle of tiles, with the matrix's edges in some of them. The two after
+    them take 128 x 192 tiles (32 columns of tiles make one round of blocks, the last one cut off) and
+    128 x 64 tiles."""
     x, w = rand((m, k), BF16, 14), rand((n, k), BF16, 15)
     want = x.double() @ w.double().T
     close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
@@ -225,11 +227,11 @@ def test_pending_sums_feed_their_consumers(ops, m):
     close(r4, full, 1e-5, "accumulate")
 
 
-@pytest.mark.parametrize("n,k", [(4112, 4096), (33000, 520)])
+@pytest.mark.parametrize("n,k", [(4112, 4096), (33000, 520), (4111, 4096)])
 def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
     """Above 16 M weights and from 4 rows on, the product for up to 16 rows stages its rows in LDS for
     four waves (N no multiple of 64: the last block has waves without weight rows; K = 520: a slab that
-    is cut off). Both forms add the same products in the same order: a row gives the same bits alone."""
+    is cut off; N = 4111: rows of partial sums that are not 16-byte aligned). Both forms add the same products in the same order: a row gives the same bits alone."""
     x, w = rand((16, k), BF16, 70), rand((n, k), BF16, 71, 0.05)
     want = x.double() @ w.double().T
     rows = {}
