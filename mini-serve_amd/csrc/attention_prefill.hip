@@ -131,7 +131,10 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
   }
 
   // Chunk c of K row R lies in slot c ^ kswz(R) of the row, chunk c of V^T row d in slot c ^ ((d >> 1) & 7).
-  auto kswz = [](int R) { return KCH == 16 ? (R & 15) : ((R >> 1) & 7); };
+  // The 16 lanes that read a chunk column together take key rows {0-3, 8-11, 16-19, 24-27} (+ 4, + 32):
+  // the rows differ in bits 0, 1, 3 and 4, and it is these that must give 16 different slots (a
+  // 256-byte row starts at bank 0; with 128-byte rows bit 0 already picks the half of the banks).
+  auto kswz = [](int R) { return KCH == 16 ? ((R & 3) | ((R >> 1) & 12)) : (((R >> 1) & 1) | ((R >> 2) & 6)); };
   // One tile's loads: wave-instruction q fills 1 KB of the stage in lane order. What does not depend on
   // the tile is worked out once: the offset of the lane's chunk within its page, and which of the
   // tile's four pages it comes from. Tiles past the last key are clamped to the last tile (what is
