@@ -367,8 +367,8 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
 // 8 rows, and what then limits large matrices). K is split over the grid so
 // that even a 1024-row matrix gives every CU several waves; each split writes float partial sums
 // P[split, M, N], which the caller's next kernel (or the reduction below) sums in ascending split
-// order. The number of splits depends on N, K and on whether M is above 16, not on M itself: a row's
-// result does not depend on the batch it is in (within the same MB).
+// order. The number of splits depends on N, K and on the class of M (up to 4, 5 to 16, above 16), not on
+// M itself: within a class a row's result does not depend on the batch it is in.
 #define SMALL_SLAB 256  // k per iteration: four steps of 64
 #define XS_STRIDE (SMALL_SLAB + 8)
 // Up to 16 rows: the shared X slab is used from this many rows and this many weights on (measured:
@@ -607,14 +607,16 @@ static int wide_tile_cols(int M, int N, int splits) {
 
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
 // its loads at once, unless that would make more waves than the chip holds a few times over (then
-// slices of several whole slabs). With up to 16 rows the partial sums are small beside the weights
-// and 32768 waves are allowed; above that 8192. At most 16 splits: the kernel that sums them up reads
-// every one. The count depends on M only through that class.
+// slices of several whole slabs). With up to 4 rows the partial sums are small beside the weights
+// and 32768 waves are allowed; above that 8192: the partial sums cost more than their bytes (at 8
+// rows a 24576 x 4096 matrix writes 12 MB of them in 16 splits, 6 % of its weights, and takes 15 %
+// longer than at 1 row; in 4 splits half of that). At most 16 splits: the kernel that sums them up
+// reads every one. The count depends on M only through its class (up to 4, 5 to 16, above 16).
 #define SMALL_MAX_SPLITS 16
 static int small_slabs_per_split(int M, int N, int K) {
   const int slabs = (K + SMALL_SLAB - 1) / SMALL_SLAB;
   const int row_blocks = (N + 15) / 16;
-  const int waves = M <= 16 ? 32768 : 8192;
+  const int waves = M <= 4 ? 32768 : 8192;
   int s = slabs;
   const int most = waves / row_blocks > 0 ? waves / row_blocks : 1;
   if (s > most) s = most;
