@@ -626,14 +626,16 @@ static int small_slabs_per_split(int M, int N, int K) {
 
 // 16 < M <= 64 and K a multiple of 64: the product runs as 64 x 64 tiles of the kernel whose slabs go
 // straight into LDS (it streams the weights faster than the four-wave small-M kernel: 2.9 -> 4.4 TB/s
-// at the 8B shapes), with K split so that about 768 blocks are in the grid, at most 16 splits and at
-// least two slabs per split.
+// at the 8B shapes), with K split so that about 768 blocks are in the grid (384 for matrices of up to
+// 16 MB, where the partial sums weigh as much as the weights: measured, 1.7 % of a batch-64 step of the
+// 0.6B shape), at most 16 splits and at least two slabs per split.
 static bool small_runs_as_tiles(int M, int K) { return M > 16 && K % BK == 0; }
 
 static int tile_slabs_per_split(int N, int K) {
   const int slabs = K / BK;
   const int cols = (N + 63) / 64;
-  int s = (768 + cols - 1) / cols;
+  const int target = (long)N * K * 2 <= (16L << 20) ? 384 : 768;
+  int s = (target + cols - 1) / cols;
   if (s > SMALL_MAX_SPLITS) s = SMALL_MAX_SPLITS;
   if (s > slabs / 2) s = slabs / 2;
   if (s < 1) s = 1;
