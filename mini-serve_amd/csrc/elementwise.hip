@@ -104,6 +104,23 @@ __global__ __launch_bounds__(NT) void rmsnorm_kernel(float* __restrict__ x, cons
 // threads per row, a thread owns up to two groups of 4 consecutive elements and moves them as vectors;
 // the partial sums of 8 splits are fetched at a time. Sums per element in ascending split order, as
 // in the kernel above.
+// acc += parts of splits s0 .. s0 + B - 1 (those below `splits`), four floats each, in ascending order;
+// the B loads are issued before the first sum.
+template <int B>
+__device__ __forceinline__ void add_splits(float4& acc, const float* __restrict__ p, int s0, int splits, size_t split_stride) {
+  float4 t[B];
+#pragma unroll
+  for (int u = 0; u < B; ++u) {
+    const bool in = s0 + u < splits;
+    t[u] = *reinterpret_cast<const float4*>(p + (size_t)(in ? s0 + u : 0) * split_stride);
+    if (!in) t[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int u = 0; u < B; ++u) {
+    acc.x += t[u].x; acc.y += t[u].y; acc.z += t[u].z; acc.w += t[u].w;
+  }
+}
+
 template <typename TW, int NT>
 __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x, const TW* __restrict__ w,
                                                             bf16* __restrict__ y, const int* __restrict__ rows, int width,
@@ -125,18 +142,14 @@ __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x,
       if (parts != nullptr) {
         const float* p = parts + row * width + i;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s0 = 0; s0 < splits; s0 += 8) {
-          float4 t[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const bool in = s0 + u < splits;
-            t[u] = *reinterpret_cast<const float4*>(p + (size_t)(in ? s0 + u : 0) * split_stride);
-            if (!in) t[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            acc.x += t[u].x; acc.y += t[u].y; acc.z += t[u].z; acc.w += t[u].w;
-          }
+        // The loads of a batch of splits go out together; few splits (a tile product's two to four) take
+        // a batch of their own size, so that no load is issued for nothing. Ascending split order always.
+        if (splits <= 2) {
+          add_splits<2>(acc, p, 0, splits, split_stride);
+        } else if (splits <= 4) {
+          add_splits<4>(acc, p, 0, splits, split_stride);
+        } else {
+          for (int s0 = 0; s0 < splits; s0 += 8) add_splits<8>(acc, p, s0, splits, split_stride);
         }
         v.x += acc.x; v.y += acc.y; v.z += acc.z; v.w += acc.w;
         if (in_place) *reinterpret_cast<float4*>(src + i) = v;
@@ -169,7 +182,7 @@ extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y
   // float32 output keeps one block shape for every batch, so that its sums are formed in one order
   // whatever the batch; bfloat16 output takes the wide block for few rows.
   const bool wide = y_is_bf16 && n_rows <= 256;
-  if (wide && width % 4 == 0 && width <= 8192 && (parts == nullptr || split_stride % 4 == 0)) {
+  if (y_is_bf16 && width % 4 == 0 && width <= 8192 && (parts == nullptr || split_stride % 4 == 0)) {
 #define LAUNCH_VEC(TW)                                                                                                  \
   if (width <= 2048)                                                                                                    \
     rmsnorm_vec4_kernel<TW, 256><<<n_rows, 256, 0, st>>>(x, (const TW*)w, (bf16*)y, rows, width, eps, parts, splits,    \
