@@ -779,15 +779,43 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
   return MS_UNSUPPORTED;  // too few tiles without a split of K
 }
 
-// Splits of K for the tile kernel when the caller takes partial sums: as many as fill the chip with
-// 128 x 128 tiles (at most 4), each at least 512 k long.
+// Splits of K for the tile kernel when the caller takes partial sums and 128 x 128 tiles alone would
+// not fill the chip. Up to 512 rows (large decode batches, short portions of prompts) the
+// product is then bound by reading the weights, and what counts is that about 512 blocks (two per CU,
+// all resident at once) share them. Matrices of up to 16 MB run as 64 x 64 tiles, K split up to 16
+// ways with at least two slabs each; larger ones as 128-row tiles, split up to 8 ways with at least
+// 512 k each (their partial sums weigh more: at 128 rows each split of a 4096-column product writes
+// 2 MB that the consumer reads again). Measured at 96 to 512 rows and the layer shapes of the 0.6B
+// and 8B models: 10 to 30 % faster than at most four splits chosen by tile count alone.
+static bool tile_small_matrix(int N, int K) { return (long)N * K * 2 <= (16L << 20); }
+
 extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   if (tiles >= 256) return 1;
-  int s = (int)((256 + tiles - 1) / tiles);
-  if (s > 4) s = 4;
-  while (s > 1 && K / s < 512) --s;
-  return s;
+  if (M > 512) {  // many rows, a narrow matrix: as many splits as fill the chip with 128 x 128 tiles, at most 4
+    int s = (int)((256 + tiles - 1) / tiles);
+    if (s > 4) s = 4;
+    while (s > 1 && K / s < 512) --s;
+    return s;
+  }
+  long want, most;
+  if (tile_small_matrix(N, K)) {
+    want = 512 / ((long)((M + 63) / 64) * ((N + 63) / 64));
+    most = K / BK / 2 < 16 ? K / BK / 2 : 16;
+  } else {
+    want = 512 / tiles;
+    most = K / 512 < 8 ? K / 512 : 8;
+  }
+  if (want > most) want = most;
+  const int allowed[8] = {16, 12, 8, 6, 4, 3, 2, 1};
+  int s = 1;
+  for (int i = 0; i < 8; ++i)
+    if (allowed[i] <= want) {
+      s = allowed[i];
+      break;
+    }
+  const int slabs = (K + BK - 1) / BK, per = (slabs + s - 1) / s;
+  return (slabs + per - 1) / per;  // no empty split
 }
 
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T

@@ -245,7 +245,8 @@ def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
     assert torch.equal(rows[16][:, :9], rows[9])
 
 
-@pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 4), (2048, 1024, 3072, 2), (300, 1000, 1100, 2), (2048, 4096, 1024, 1)])
+@pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 8), (2048, 1024, 3072, 2), (300, 1000, 1100, 6), (2048, 4096, 1024, 1),
+                                          (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6)])
 def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
     x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
     want = x.double() @ w.double().T
