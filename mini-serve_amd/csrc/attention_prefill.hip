@@ -22,6 +22,11 @@
 // shortens that chain.
 // blockIdx.x = tile * Hkv + kvh: with 8 KV heads every KV head stays on one XCD and its tiles share
 // that XCD's L2.
+//
+// A batch with few tiles (one short prompt) leaves the chip to the deepest tile's chain of iterations,
+// which runs on alone when every other block is done. The host may therefore hand a tile's keys out in
+// parts: an entry then names a range of key tiles and a slot, the block leaves its running maximum,
+// sum and unnormalised output there, and a second kernel merges a tile's parts in ascending order.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -63,7 +68,9 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos,
-    bf16* __restrict__ out, int Hq, int Hkv, float scale, int window) {
+    bf16* __restrict__ out, int Hq, int Hkv, float scale, int window, const int* __restrict__ tile_key_begin,
+    const int* __restrict__ tile_key_end, const int* __restrict__ tile_slot, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
   constexpr int NT = 256 * KSPLIT, NW = NT / WAVE;
   constexpr int KK = D / 32, DB = D / 16;
   constexpr int ROWS = 64 * NQ;     // query rows per block
@@ -173,8 +180,12 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
   };
 
   const float scale2 = scale * 1.44269504088896340736f;  // scores in units of log2: exp2 is one instruction
-  const int t_first = (kv_lo / TK) * TK;
-  const int n_tiles = (last_pos - t_first) / TK + 1;
+  // The key tiles this block visits: all the tile's rows may see, or the part the host names (in units
+  // of key tiles from position 0; the host leaves no part empty).
+  const int slot = tile_slot ? tile_slot[tile] : -1;
+  const int t_first = max((kv_lo / TK) * TK, tile_key_begin ? tile_key_begin[tile] * TK : 0);
+  const int key_last = tile_key_end ? min(last_pos, tile_key_end[tile] * TK - 1) : last_pos;
+  const int n_tiles = (key_last - t_first) / TK + 1;
   // Issue order: page ids of tile m + 1, then the loads of tile m. At the top of iteration n the loads
   // of tiles n + 1 .. n + STAGES - 2 may still be in flight, those of tile n must have landed.
   i32x4 pages_next = tile_pages(table, t_first, last_pos);
@@ -339,6 +350,22 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
   }
 
   // o[b][db][i] = O[row r of block b][d = db * 16 + 4 g + i]
+  if (slot >= 0) {
+    // A part of the tile's keys: maximum, sum and unnormalised output of every row go to the slot.
+    const size_t base = ((size_t)slot * Hkv + kvh) * ROWS;
+#pragma unroll
+    for (int b = 0; b < NQ; ++b) {
+      const int row = rg * WROWS + b * 16 + r;
+      float* po = part_o + (base + row) * D + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(po + db * 16) = o[b][db];
+      if (g == 0) {
+        part_ml[(base + row) * 2] = m_run[b];
+        part_ml[(base + row) * 2 + 1] = l_run[b];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < NQ; ++b) {
     const float inv = 1.f / l_run[b];
@@ -357,6 +384,58 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
   }
 }
 
+// Merges the parts of the tiles whose keys were handed out in parts: grid (merged tiles, Hkv). A tile's
+// parts lie in consecutive slots, in ascending order of their keys, and are added in that order. A part
+// in which a row saw no key (behind its window) has maximum -inf and adds nothing.
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const int* __restrict__ merge_first,
+                                                                 const int* __restrict__ merge_count,
+                                                                 const int* __restrict__ merge_slot,
+                                                                 const int* __restrict__ merge_parts,
+                                                                 const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                                                 int Hq, int Hkv, int rows) {
+  const int t = blockIdx.x, kvh = blockIdx.y;
+  const int G = Hq / Hkv;
+  const int first = merge_first[t], count = merge_count[t], slot0 = merge_slot[t], parts = merge_parts[t];
+  const int used = min(count * G, (rows / G) * G);  // rows of the tile that hold a token's head
+  for (int idx = threadIdx.x; idx < used * (D / 4); idx += 256) {
+    const int row = idx / (D / 4), d = (idx % (D / 4)) * 4;
+    float m = -INFINITY;
+    for (int p = 0; p < parts; ++p) m = fmaxf(m, part_ml[(((size_t)(slot0 + p) * Hkv + kvh) * rows + row) * 2]);
+    float l = 0.f;
+    floatx4 o = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < parts; ++p) {
+      const size_t at = ((size_t)(slot0 + p) * Hkv + kvh) * rows + row;
+      const float mp = part_ml[at * 2];
+      const float f = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - m);
+      l += part_ml[at * 2 + 1] * f;
+      const floatx4 v = *reinterpret_cast<const floatx4*>(part_o + at * D + d);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] += v[i] * f;
+    }
+    const float inv = 1.f / l;
+    bf16x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<bf16>(o[i] * inv);
+    *reinterpret_cast<bf16x4*>(out + ((size_t)(first + row / G) * Hq + kvh * G + row % G) * D + d) = v;
+  }
+}
+
+// What the host adds when it hands tiles' keys out in parts (all null / 0 otherwise).
+struct PrefillParts {
+  const int* key_begin;    // per entry: first key tile
+  const int* key_end;      // per entry: one past its last key tile
+  const int* slot;         // per entry: where its partial result goes, or -1: it is the whole tile
+  float* part_o;           // [slots, Hkv, rows per tile, D]
+  float* part_ml;          // [slots, Hkv, rows per tile, 2]
+  const int* merge_first;  // per merged tile: first token, token count, first slot, number of parts
+  const int* merge_count;
+  const int* merge_slot;
+  const int* merge_parts;
+  int merges;
+};
+
 template <int D, int NQ, int KSPLIT, int STAGES>
 constexpr int prefill_lds_bytes() {
   constexpr int tiles = STAGES * (TK * D * 2 + D * TK * 2);
@@ -367,7 +446,8 @@ constexpr int prefill_lds_bytes() {
 template <int D, int NQ, int KSPLIT, int STAGES, int BLOCKS_PER_CU>
 static int launch_prefill(unsigned grid, const bf16* q, int q_stride, const bf16* kc, const bf16* vc, const int* block_table,
                           int table_width, const int* tile_first, const int* tile_count, const int* token_row,
-                          const int* pos, bf16* out, int Hq, int Hkv, float scale, int window, hipStream_t st) {
+                          const int* pos, bf16* out, int Hq, int Hkv, float scale, int window, PrefillParts pp,
+                          hipStream_t st) {
   constexpr int lds = prefill_lds_bytes<D, NQ, KSPLIT, STAGES>();
   static_assert(lds * BLOCKS_PER_CU <= 160 * 1024, "LDS of the blocks that share a CU");
   static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
@@ -379,28 +459,32 @@ static int launch_prefill(unsigned grid, const bf16* q, int q_stride, const bf16
   }
   attn_prefill_kernel<D, NQ, KSPLIT, STAGES, BLOCKS_PER_CU><<<grid, 256 * KSPLIT, lds, st>>>(q, q_stride, kc, vc, block_table, table_width,
                                                                               tile_first, tile_count, token_row, pos, out,
-                                                                              Hq, Hkv, scale, window);
+                                                                              Hq, Hkv, scale, window, pp.key_begin, pp.key_end,
+                                                                              pp.slot, pp.part_o, pp.part_ml);
+  if (pp.merges > 0)
+    attn_prefill_merge_kernel<D><<<dim3(pp.merges, Hkv), 256, 0, st>>>(pp.merge_first, pp.merge_count, pp.merge_slot,
+                                                                       pp.merge_parts, pp.part_o, pp.part_ml, out, Hq, Hkv,
+                                                                       64 * NQ);
   return launch_status();
 }
 #define PREFILL_ARGS                                                                                                    \
   (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, \
-      pos, (bf16*)out, Hq, Hkv, scale, window, st
+      pos, (bf16*)out, Hq, Hkv, scale, window, pp, st
 
 // Tokens per tile for a group of G query heads per KV head and `rows` query rows per block.
 extern "C" int ms_attention_prefill_tile_tokens(int G, int rows) { return G >= 1 && G <= rows ? rows / G : 0; }
 
 // rows_per_tile: 128 (large batches of tiles: least traffic per product) or 64 (each wave then takes
 // half of every key tile: shortest chain per tile).
-extern "C" int ms_attention_prefill_bf16(const void* q, int q_stride, const void* kc, const void* vc,
-                                         const int* block_table, int table_width, const int* tile_first,
-                                         const int* tile_count, int tiles, int rows_per_tile, const int* token_row,
-                                         const int* pos, void* out, int Hq, int Hkv, int D, int page_size, float scale,
-                                         int window, hipStream_t st) {
+static int prefill_dispatch(const void* q, int q_stride, const void* kc, const void* vc, const int* block_table,
+                            int table_width, const int* tile_first, const int* tile_count, int tiles, int rows_per_tile,
+                            const int* token_row, const int* pos, void* out, int Hq, int Hkv, int D, int page_size,
+                            float scale, int window, PrefillParts pp, hipStream_t st) {
   if (tiles <= 0) return MS_OK;
   if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 64 || window < 0 || table_width <= 0 || table_width % 4 ||
       q_stride < Hq * D || q_stride % 8 || (long long)tiles * Hkv > 2147483647LL ||
-      (rows_per_tile != 64 && rows_per_tile != 128))
+      (rows_per_tile != 64 && rows_per_tile != 128) || Hkv > 65535)
     return MS_BAD_ARG;
   const unsigned grid = (unsigned)tiles * Hkv;
   // Two stages were as fast as four in every shape tried (the loop is bound by its instructions, not
@@ -409,4 +493,41 @@ extern "C" int ms_attention_prefill_bf16(const void* q, int q_stride, const void
   if (D == 128) return launch_prefill<128, 1, 2, 2, 2>(grid, PREFILL_ARGS);
   if (rows_per_tile == 128) return launch_prefill<64, 2, 1, 2, 2>(grid, PREFILL_ARGS);
   return launch_prefill<64, 1, 2, 2, 2>(grid, PREFILL_ARGS);
+}
+
+extern "C" int ms_attention_prefill_bf16(const void* q, int q_stride, const void* kc, const void* vc,
+                                         const int* block_table, int table_width, const int* tile_first,
+                                         const int* tile_count, int tiles, int rows_per_tile, const int* token_row,
+                                         const int* pos, void* out, int Hq, int Hkv, int D, int page_size, float scale,
+                                         int window, hipStream_t st) {
+  return prefill_dispatch(q, q_stride, kc, vc, block_table, table_width, tile_first, tile_count, tiles, rows_per_tile,
+                          token_row, pos, out, Hq, Hkv, D, page_size, scale, window, PrefillParts{}, st);
+}
+
+// The same with tiles' keys handed out in parts. `plan` holds, as consecutive int arrays on the device:
+// per entry (entries of them) first token, token count, first key tile, end key tile, slot (-1: the
+// entry is a whole tile); then per merged tile (merges of them) first token, token count, first slot,
+// number of parts. part_o holds slots * Hkv * rows_per_tile * D floats, part_ml slots * Hkv *
+// rows_per_tile * 2. Only for layers without a window: the parts count key tiles from position 0.
+extern "C" int ms_attention_prefill_parts_bf16(const void* q, int q_stride, const void* kc, const void* vc,
+                                               const int* block_table, int table_width, const int* plan, int entries,
+                                               int merges, float* part_o, float* part_ml, int rows_per_tile,
+                                               const int* token_row, const int* pos, void* out, int Hq, int Hkv, int D,
+                                               int page_size, float scale, hipStream_t st) {
+  if (entries <= 0) return MS_OK;
+  if (plan == nullptr || merges < 0 || (merges > 0 && (!part_o || !part_ml))) return MS_BAD_ARG;
+  PrefillParts pp;
+  pp.key_begin = plan + 2 * (size_t)entries;
+  pp.key_end = plan + 3 * (size_t)entries;
+  pp.slot = plan + 4 * (size_t)entries;
+  pp.part_o = part_o;
+  pp.part_ml = part_ml;
+  const int* m = plan + 5 * (size_t)entries;
+  pp.merge_first = m;
+  pp.merge_count = m + merges;
+  pp.merge_slot = m + 2 * (size_t)merges;
+  pp.merge_parts = m + 3 * (size_t)merges;
+  pp.merges = merges;
+  return prefill_dispatch(q, q_stride, kc, vc, block_table, table_width, plan, plan + entries, entries, rows_per_tile,
+                          token_row, pos, out, Hq, Hkv, D, page_size, scale, 0, pp, st);
 }

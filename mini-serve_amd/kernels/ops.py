@@ -47,6 +47,9 @@ _SIGNATURES = {
                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
                                   _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    "ms_attention_prefill_parts_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void,
+                                        _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                        _c_void],
     "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_sample_scratch_bytes": [_c_int],
@@ -578,7 +581,17 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
         # give short chains and more blocks. The latter until 128-row blocks alone fill the chip twice over.
         n_prefill = t - n_dec
         rows = 128 if (group > 64 or -(-n_prefill // (128 // group)) * num_kv_heads >= PREFILL_BIG_BLOCKS) else 64
-        first, count, tiles = batch.prefill_tiles(lib.ms_attention_prefill_tile_tokens(group, rows))
+        tile_tokens = lib.ms_attention_prefill_tile_tokens(group, rows)
+        plan = _prefill_parts_plan(batch, tile_tokens, num_kv_heads, rows * head_dim * 4) if window == 0 else None
+        if plan is not None:
+            part_o = torch.empty((plan.slots * num_kv_heads * rows * head_dim,), dtype=F32, device=qkv.device)
+            part_ml = torch.empty((plan.slots * num_kv_heads * rows * 2,), dtype=F32, device=qkv.device)
+            _check(lib.ms_attention_prefill_parts_bf16(
+                qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, plan.table.data_ptr(),
+                plan.entries, plan.merges, part_o.data_ptr(), part_ml.data_ptr(), rows, *meta, num_heads, num_kv_heads,
+                head_dim, page, float(scale), _stream()), "attention_prefill_parts")
+            return out
+        first, count, tiles = batch.prefill_tiles(tile_tokens)
         _check(lib.ms_attention_prefill_bf16(
             qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(),
             tiles, rows, *meta, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()),
@@ -601,6 +614,88 @@ def build_prefill_tiles(row_lens, row_starts, tile_tokens: int, device):
     host = torch.tensor([[f for _, f, _ in tiles], [c for _, _, c in tiles]], dtype=I32)
     dev = host.to(device, non_blocking=True)
     return dev[0], dev[1], len(tiles)
+
+
+PREFILL_KEY_TILE = 64        # keys per iteration of the prefill attention kernel
+PREFILL_RESIDENT_BLOCKS = 512  # blocks of it the chip holds at once (two per CU)
+PREFILL_MIN_PART = 4         # key tiles: no part is made shorter than this
+PREFILL_PARTS_LAUNCH_US = 8.0  # what the merge kernel costs beside the bytes it moves
+PREFILL_PARTS_MARGIN = 1.5   # parts are made where they save this many times what they cost
+
+
+class PrefillPartsPlan:
+    """Tiles of new tokens whose keys are handed out in parts. ``table``: int32 on the device, per entry
+    first token, token count, first key tile, end key tile, slot (-1: a whole tile), heaviest entry
+    first; then per merged tile first token, token count, first slot, number of parts."""
+
+    __slots__ = ("table", "entries", "merges", "slots")
+
+    def __init__(self, table, entries, merges, slots):
+        self.table, self.entries, self.merges, self.slots = table, entries, merges, slots
+
+
+def plan_prefill_parts(row_lens, row_starts, tile_tokens: int, kv_heads: int, part_bytes: int = 64 * 128 * 4):
+    """Host part of ``PrefillPartsPlan``: ``(entries, merges)`` as lists of tuples, or None where
+    whole tiles do as well. A step takes as long as its deepest tile's chain of key tiles (about 1.2 us
+    each for a block on its own) or as long as all key tiles take the chip (about 2.4 us for each
+    resident block's), whichever is longer. Where the chain is the longer by far (a short portion
+    deep into a long sequence), the keys of tiles deeper than the chip's fair share (all key tiles /
+    resident blocks) are cut into equal parts no longer than that share. The parts cost a second
+    kernel and ``part_bytes`` written and read per part and KV head, so whole tiles stay unless the
+    shorter chain saves half as much again as that (measured: one 2,048-token prompt is slower in
+    parts, a 512-token portion behind 16,000 cached tokens a quarter faster)."""
+    tiles = []
+    t = 0
+    for n, s in zip(row_lens, row_starts):
+        if n > 1:
+            for a in range(0, n, tile_tokens):
+                c = min(tile_tokens, n - a)
+                tiles.append(((s + a + c - 1) // PREFILL_KEY_TILE + 1, t + a, c))
+        t += n
+    if not tiles or len(tiles) * kv_heads >= 2 * PREFILL_RESIDENT_BLOCKS:
+        return None
+    total = sum(d for d, _, _ in tiles) * kv_heads
+    share = max(PREFILL_MIN_PART, -(-total // PREFILL_RESIDENT_BLOCKS))
+    deepest = max(d for d, _, _ in tiles)
+    if deepest <= share:
+        return None
+    slots = sum(-(-d // share) for d, _, _ in tiles if d > share)
+    busy_us = 2.4 * total / PREFILL_RESIDENT_BLOCKS
+    saved_us = 1.2 * deepest - max(1.2 * share, busy_us)
+    cost_us = PREFILL_PARTS_LAUNCH_US + 2 * slots * kv_heads * part_bytes / 3e6
+    if saved_us <= PREFILL_PARTS_MARGIN * cost_us:
+        return None
+    entries, merges, slot = [], [], 0
+    for depth, first, count in tiles:
+        parts = -(-depth // share)
+        if parts == 1:
+            entries.append((first, count, 0, depth, -1))
+            continue
+        per = -(-depth // parts)
+        parts = -(-depth // per)
+        merges.append((first, count, slot, parts))
+        for p in range(parts):
+            entries.append((first, count, p * per, min(depth, (p + 1) * per), slot))
+            slot += 1
+    entries.sort(key=lambda e: e[2] - e[3])  # most key tiles first
+    return entries, merges
+
+
+def _prefill_parts_plan(batch, tile_tokens: int, kv_heads: int, part_bytes: int):
+    memo = getattr(batch, "memo", None)
+    key = ("prefill_parts", tile_tokens, kv_heads, part_bytes)
+    if memo is not None and key in memo:
+        return memo[key]
+    plan = None
+    made = plan_prefill_parts(batch.row_lens, batch.row_starts_host, tile_tokens, kv_heads, part_bytes)
+    if made is not None:
+        entries, merges = made
+        flat = [e[i] for i in range(5) for e in entries] + [m[i] for i in range(4) for m in merges]
+        table = torch.tensor(flat, dtype=I32).to(batch.positions.device, non_blocking=True)
+        plan = PrefillPartsPlan(table, len(entries), len(merges), sum(m[3] for m in merges))
+    if memo is not None:
+        memo[key] = plan
+    return plan
 
 
 # ------------------------------------------------------------------------------------- sampling

@@ -479,10 +479,28 @@ def test_decode_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost)
         (16, 8, 128, [150, 30], [0, 500], 40, (0, 149 - 39)),         # a window: its first key stands out
         (16, 8, 128, [130], [300], 200, (0, 230)),                    # a window wider than the tile
         (6, 6, 64, [300], [0], 17, None),                             # a window narrower than a key tile
+        (16, 8, 128, [700], [0], 0, (0, 100)),                        # deep tiles' keys in parts: a key of an early part
+        (16, 8, 128, [300, 1], [900, 50], 0, (0, 1199 - 70)),         # parts beside a decode row: a key of the last but one part
+        (8, 2, 64, [500, 40], [0, 0], 0, (0, 3)),                     # head size 64, whole tiles beside tiles in parts
+        (16, 8, 128, [64, 1], [6000, 9], 0, (0, 4000)),               # a short portion far into a sequence: parts by the host's own rule
     ],
 )
-def test_prefill_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost):
+@pytest.mark.parametrize("parts", ["host rule", "wherever possible"])
+def test_prefill_attention_bf16(ops, monkeypatch, hq, hkv, d, lens_new, starts, window, boost, parts):
+    """``parts``: the keys of deep tiles are handed out in parts where the host's estimate says it pays, or
+    (second run) wherever a tile is deeper than the shortest part, so that small cases take that path too."""
+    if parts == "wherever possible":
+        monkeypatch.setattr(ops, "PREFILL_PARTS_LAUNCH_US", -1e9)
     attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=40, boost=boost)
+
+
+def test_prefill_attention_parts_are_taken(ops, monkeypatch):
+    """The cases above do reach the kernel that merges parts: the plan of a short portion far into a
+    sequence has parts under the host's own rule, and forcing them changes results by rounding only."""
+    assert ops.plan_prefill_parts([64, 1], [6000, 9], 32, 8) is not None
+    assert ops.plan_prefill_parts([700], [0], 32, 8) is None
+    monkeypatch.setattr(ops, "PREFILL_PARTS_LAUNCH_US", -1e9)
+    assert ops.plan_prefill_parts([700], [0], 32, 8) is not None
 
 
 @pytest.mark.parametrize(
