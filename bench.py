@@ -41,7 +41,10 @@ def main() -> int:
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill measurement")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps eagerly")
-    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiling)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="tokens of the timed prefill step")
+    ap.add_argument("--prefill-cached", type=int, default=0,
+                    help="tokens of the same sequence already in the cache when the timed step runs (fed untimed, 2,048 a step)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -135,12 +138,14 @@ def main() -> int:
         # Prefill of one 2,048-token prompt in one step (logits at the last position).
         from miniserve_amd.engine.runner import ModelRunner
 
-        T = 2048
-        runner = ModelRunner(model, kv_pool_tokens=4 * T, max_running=4)
+        T, C = args.prefill_tokens, args.prefill_cached
+        runner = ModelRunner(model, kv_pool_tokens=4 * T + C + 64, max_running=4)
         times = []
         for i in range(4):
             rc = runner.acquire()
             ids = prompts(1, T)[0]
+            for at in range(0, C, 2048):
+                runner.step([StepRow(rc, prompts(1, min(2048, C - at))[0], [])])
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             runner.step([StepRow(rc, ids, [T - 1])])
@@ -151,11 +156,13 @@ def main() -> int:
         L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
         Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
         linear = 2 * T * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I) + 2 * H * vocab
-        attn = 2 * T * T * D * Hq * L  # causal: QK^T and PV over half the square each
+        attn = 2 * T * (T + 2 * C) * D * Hq * L  # causal: QK^T and PV over half the square each, and over the cached keys
         flops = linear + attn
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         out["prefill"] = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
                           "frac": round(flops / pre / peak, 4)}
+        if C:
+            out["prefill"]["cached"] = C
         del runner
         points = {}
         for b, steps in ((1, 64), (64, 24)) if not args.prefill_only else ():
