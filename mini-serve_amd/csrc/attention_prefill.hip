@@ -384,7 +384,8 @@ __global__ __launch_bounds__(256 * KSPLIT, BLOCKS_PER_CU * KSPLIT) void attn_pre
   }
 }
 
-// Merges the parts of the tiles whose keys were handed out in parts: grid (merged tiles, Hkv). A tile's
+// Merges the parts of the tiles whose keys were handed out in parts: grid (merged tiles, Hkv, groups of
+// 16 rows). A tile's
 // parts lie in consecutive slots, in ascending order of their keys, and are added in that order. A part
 // in which a row saw no key (behind its window) has maximum -inf and adds nothing.
 template <int D>
@@ -399,7 +400,8 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const int* __re
   const int G = Hq / Hkv;
   const int first = merge_first[t], count = merge_count[t], slot0 = merge_slot[t], parts = merge_parts[t];
   const int used = min(count * G, (rows / G) * G);  // rows of the tile that hold a token's head
-  for (int idx = threadIdx.x; idx < used * (D / 4); idx += 256) {
+  const int row_end = min(used, (int)(blockIdx.z + 1) * 16);
+  for (int idx = blockIdx.z * 16 * (D / 4) + threadIdx.x; idx < row_end * (D / 4); idx += 256) {
     const int row = idx / (D / 4), d = (idx % (D / 4)) * 4;
     float m = -INFINITY;
     for (int p = 0; p < parts; ++p) m = fmaxf(m, part_ml[(((size_t)(slot0 + p) * Hkv + kvh) * rows + row) * 2]);
@@ -462,7 +464,7 @@ static int launch_prefill(unsigned grid, const bf16* q, int q_stride, const bf16
                                                                               Hq, Hkv, scale, window, pp.key_begin, pp.key_end,
                                                                               pp.slot, pp.part_o, pp.part_ml);
   if (pp.merges > 0)
-    attn_prefill_merge_kernel<D><<<dim3(pp.merges, Hkv), 256, 0, st>>>(pp.merge_first, pp.merge_count, pp.merge_slot,
+    attn_prefill_merge_kernel<D><<<dim3(pp.merges, Hkv, 4 * NQ), 256, 0, st>>>(pp.merge_first, pp.merge_count, pp.merge_slot,
                                                                        pp.merge_parts, pp.part_o, pp.part_ml, out, Hq, Hkv,
                                                                        64 * NQ);
   return launch_status();
