@@ -85,3 +85,49 @@ def test_random_configuration(seed, medium, tmp_path):
             for i in ends:
                 runner.release(live.pop(i))
         assert runner.cache.idle, "pages were not all given back"
+
+
+@pytest.mark.parametrize("name", ("tinyD", "tinyE"))
+def test_portions_with_keys_in_parts(name, tmp_path, monkeypatch):
+    """Portions of prompts beside single tokens with the prefill attention forced to hand the keys of
+    every tile deeper than four key tiles out in parts (the host's own rule does so only far into long
+    sequences): the step function's logits still follow the plain implementation. tinyD has head
+    size 64, tinyE head size 128 and a windowed layer, which keeps whole tiles."""
+    from miniserve_amd.engine.batch import StepRow
+    from miniserve_amd.engine.runner import ModelRunner
+    from miniserve_amd.kernels import ops
+    from miniserve_amd.loading import load_model
+    from models import make_folder
+
+    monkeypatch.setattr(ops, "PREFILL_PARTS_LAUNCH_US", -1e9)
+    folder = make_folder(tmp_path, name)
+    pcfg, w = read_model_folder(folder)
+    rng = np.random.default_rng(5)
+    lengths = [700, 330, 90]
+    reqs = [rng.integers(0, pcfg["vocab_size"], size=n).tolist() for n in lengths]
+    want = [P.logits(pcfg, w, ids) for ids in reqs]
+    runner = ModelRunner(load_model(folder, "bfloat16", "cuda:0"), page_size=16, kv_pool_tokens=1280, max_running=4)
+    rcs = [runner.acquire() for _ in reqs]
+    fed = [0, 0, 0]
+    taken = 0
+    for portion in (300, 64, 200, 33, 128, 2, 400):
+        rows, spans = [], []
+        for i, n in enumerate(lengths):
+            k = min(portion if i != 2 else 1, n - fed[i])  # the third request goes one token at a time
+            if k > 0:
+                rows.append(StepRow(rcs[i], reqs[i][fed[i] : fed[i] + k], list(range(k))))
+                spans.append((i, fed[i], k))
+                fed[i] += k
+        if not rows:
+            break
+        plan = ops.plan_prefill_parts([k for _, _, k in spans], [s for _, s, _ in spans], 32, 1)
+        taken += plan is not None
+        got = runner.step(rows).float().cpu().numpy()
+        at = 0
+        for i, s, k in spans:
+            check_logits(got[at : at + k], want[i][s : s + k], "bfloat16", f"{name} request {i} tokens {s}..{s + k}")
+            at += k
+    assert taken >= 3, "the steps were meant to have tiles deep enough to be cut"
+    for rc in rcs:
+        runner.release(rc)
+    assert runner.cache.idle
