@@ -678,7 +678,6 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
   // Without a shared X slab the waves of a block have nothing in common: single-wave blocks spread
-  // evenly over the CUs.
   // evenly over the CUs. Both forms add up the same products in the same order.
   const bool shared = M >= SMALL_SHARED_MIN_ROWS && (long)N * K >= SMALL_SHARED_MIN_WEIGHTS;
   if (M <= 16 && !shared) gemm_bf16_small_kernel<1, false><<<(unsigned)wave_blocks, WAVE, 0, st>>>(x, w, partials, M, N, K, ldx, per, splits);
