@@ -87,6 +87,53 @@ def cmd_stress(args) -> int:
     return 0 if finished == len(reqs) and eng.runner.cache.idle else 1
 
 
+def cmd_roofline(args) -> int:
+    """What this GPU gives beside its published peaks, measured with the engine's own kernels: the rate
+    of a streaming read and of a streaming copy over ``--mib`` MiB (the reference measures both at
+    1 GiB, bench/roofline.py:85-121), and the bfloat16 matrix product's rate at n = 4096 and 8192
+    (bench/roofline.py:184-198). Times are medians of ``--repeats`` runs by device events."""
+    import torch
+
+    from .kernels import ops
+
+    dev = torch.device(args.device)
+    torch.cuda.set_device(dev)
+
+    def median_ms(fn):
+        fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(args.repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        return sorted(times)[len(times) // 2]
+
+    n = args.mib << 20
+    src = torch.empty((n,), dtype=torch.uint8, device=dev)
+    dst = torch.empty((n,), dtype=torch.uint8, device=dev)
+    src.random_(0, 256)
+    report = {"device": torch.cuda.get_device_name(dev), "mib": args.mib, "repeats": args.repeats}
+    with ops.stream_scope():
+        report["read_GBps"] = round(n / median_ms(lambda: ops.measure_read(src, args.blocks)) / 1e6, 1)
+        report["copy_GBps"] = round(2 * n / median_ms(lambda: ops.measure_copy(src, dst, args.blocks)) / 1e6, 1)
+        assert torch.equal(src[: 1 << 20], dst[: 1 << 20]) and torch.equal(src[-(1 << 20) :], dst[-(1 << 20) :])
+        del src, dst
+        gemm = {}
+        for size in (4096, 8192):
+            x = torch.randn((size, size), device=dev).to(torch.bfloat16)
+            w = torch.randn((size, size), device=dev).to(torch.bfloat16)
+            ms = median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16))
+            gemm[str(size)] = round(2 * size**3 / ms / 1e9, 1)
+        report["gemm_bf16_TFLOPs"] = gemm
+    report["published"] = {"hbm_GBps": 8000.0, "bf16_TFLOPs": 2500.0}
+    print(json.dumps(report))
+    return 0
+
+
 def main(argv=None) -> int:
     from .engine.cli import add_engine_args
 
@@ -118,6 +165,13 @@ def main(argv=None) -> int:
     s.add_argument("--top-p", type=float, default=1.0)
     s.add_argument("--max-steps", type=int, default=100000)
     s.set_defaults(fn=cmd_stress)
+
+    r = sub.add_parser("roofline", help="measured read / copy bandwidth and bfloat16 matrix-product rate of this GPU")
+    r.add_argument("--device", default="cuda:0")
+    r.add_argument("--mib", type=int, default=1024, help="size of the buffers that are read and copied")
+    r.add_argument("--blocks", type=int, default=4096, help="blocks of the streaming kernels")
+    r.add_argument("--repeats", type=int, default=9)
+    r.set_defaults(fn=cmd_roofline)
 
     w = sub.add_parser("random-weights", help="write a model folder with random weights")
     w.add_argument("rest", nargs=argparse.REMAINDER)

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_sample_scratch_bytes": [_c_int],
+    "ms_measure_read": [_c_void, _c_ll, _c_int, _c_void, _c_void],
+    "ms_measure_copy": [_c_void, _c_void, _c_ll, _c_int, _c_void],
 }
 
 
@@ -724,3 +726,28 @@ def sample_rows(logits, temperature=None, top_p=None, seed=None, counter=None) -
     _check(lib.ms_sample_rows(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
                               _ptr(counter), scratch.data_ptr(), out.data_ptr(), _stream()), "sample_rows")
     return out
+
+
+# ------------------------------------------------------------------------------------- measurement
+
+
+def measure_read(buffer: torch.Tensor, blocks: int = 4096) -> torch.Tensor:
+    """Streams ``buffer`` (contiguous, a multiple of 16 bytes) through ``blocks`` blocks once and
+    returns their checksums ``int32 [blocks]``: the read half of the memory system's rate."""
+    if not buffer.is_cuda or not buffer.is_contiguous():
+        raise ValueError("measure_read takes a contiguous tensor on the GPU")
+    out = torch.empty((blocks,), dtype=I32, device=buffer.device)
+    _check(library().ms_measure_read(buffer.data_ptr(), buffer.numel() * buffer.element_size(), blocks, out.data_ptr(),
+                                     _stream()), "measure_read")
+    return out
+
+
+def measure_copy(src: torch.Tensor, dst: torch.Tensor, blocks: int = 4096) -> None:
+    """``dst[:] = src`` as a streaming copy of ``blocks`` blocks (both contiguous, same size, a multiple
+    of 16 bytes)."""
+    if not (src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("measure_copy takes contiguous tensors on the GPU")
+    n = src.numel() * src.element_size()
+    if n != dst.numel() * dst.element_size():
+        raise ValueError("source and destination differ in size")
+    _check(library().ms_measure_copy(src.data_ptr(), dst.data_ptr(), n, blocks, _stream()), "measure_copy")

@@ -34,7 +34,7 @@ def test_build_finds_every_source():
     from miniserve_amd.kernels import build
 
     names = {s.name for s in build.hip_sources()}
-    assert {"attention.hip", "attention_decode.hip", "attention_prefill.hip", "elementwise.hip", "gemm_bf16.hip",
+    assert {"attention.hip", "attention_decode.hip", "attention_prefill.hip", "elementwise.hip", "gemm_bf16.hip", "measure.hip",
             "gemm_f32.hip", "sampling.hip"} <= names
     assert [s.name for s in build.cpp_sources()] == ["block_core.cpp"]
     assert "-packed-fp32-ops" in build.HIP_FLAGS, "packed float32 instructions stay off"

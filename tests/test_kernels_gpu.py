@@ -640,3 +640,21 @@ def test_sampling_frequencies_follow_softmax(ops):
         freq = torch.bincount(toks.long(), minlength=8).double().cpu() / n
         want = torch.softmax(base.double().cpu() / temp, 0)
         assert float((freq - want).abs().max()) < 0.01
+
+
+# ------------------------------------------------------------------------------------------ measuring kernels
+
+
+@pytest.mark.parametrize("vectors,blocks", [(1, 1), (255, 3), (256 * 8 * 5, 4), (256 * 8 * 5 + 77, 4), (100000, 64), (2048 * 9 + 1, 7)])
+def test_streaming_read_and_copy_touch_every_vector_once(ops, vectors, blocks):
+    """The kernels behind the measured bandwidths: the read's checksums, xor-ed, equal the xor of the
+    whole buffer (every 16-byte vector seen exactly once, partial last chunk included), and the copy
+    reproduces its source and nothing beyond."""
+    g = torch.Generator().manual_seed(vectors)
+    src = torch.randint(-(2**31), 2**31 - 1, (vectors * 4,), generator=g, dtype=torch.int64).to(torch.int32).to(DEV)
+    sums = ops.measure_read(src, blocks).cpu().numpy().astype(np.uint32)
+    want = np.bitwise_xor.reduce(src.cpu().numpy().astype(np.uint32))
+    assert np.bitwise_xor.reduce(sums) == want
+    dst = torch.full((vectors * 4 + 8,), 7, dtype=torch.int32, device=DEV)
+    ops.measure_copy(src, dst[: vectors * 4], blocks)
+    assert torch.equal(dst[: vectors * 4], src) and bool((dst[vectors * 4 :] == 7).all())
