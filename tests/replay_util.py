@@ -4,7 +4,6 @@ acknowledged by ``done <step>``; logits are read from the files it writes."""
 from __future__ import annotations
 
 import json
-import os
 import subprocess
 import sys
 from pathlib import Path

@@ -4,7 +4,6 @@ in steps of 16, odd head counts and groups, rows that do not fill a tile."""
 
 from __future__ import annotations
 
-import math
 
 import numpy as np
 import pytest
