@@ -215,9 +215,19 @@ __device__ __forceinline__ void banded(int t, int rows, int cols, int band_cols,
 // activations, which is what counts when the weight matrix is the smaller operand.
 __device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int col_tiles, int xcd_rows, int band_cols) {
   const int tiles = row_tiles * col_tiles;
-  const int t = block % tiles;
+  const int splits = gridDim.x / tiles;
   TileId id;
-  id.split = block / tiles;
+  int t;
+  if (row_tiles == 1 && splits > 1) {
+    // One row of tiles with K split (a product bound by streaming its weights): the split index runs
+    // fastest, so that neighbouring blocks read neighbouring k ranges of the same weight rows rather
+    // than the same k range of rows that lie a power of two apart (2-3 % faster at 32 to 128 rows).
+    id.split = block % splits;
+    t = block / splits;
+  } else {
+    t = block % tiles;
+    id.split = block / tiles;
+  }
   if (xcd_rows == 0) {
     banded(t, row_tiles, col_tiles, band_cols, id.m, id.n);
     return id;
