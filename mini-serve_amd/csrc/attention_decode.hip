@@ -174,13 +174,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
     const bf16* k0 = kc + (((size_t)kp * Hkv + kvh) * PAGE + kt) * D + g * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      t.ka[kk] = *reinterpret_cast<const bf16x8*>(k0 + kk * 32);
-      t.kb[kk] = *reinterpret_cast<const bf16x8*>(k0 + 4 * D + kk * 32);
+      t.ka[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(k0 + kk * 32));
+      t.kb[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(k0 + 4 * D + kk * 32));
     }
     // V^T operand: element d = db * 16 + r, tokens 8 (g % 2) .. + 7 of page g / 2.
     const bf16* v0 = vc + (((size_t)(g < 2 ? p0 : p1) * Hkv + kvh) * D + r) * PAGE + (g % 2) * 8;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) t.v[db] = *reinterpret_cast<const bf16x8*>(v0 + (size_t)db * 16 * PAGE);
+    for (int db = 0; db < DB; ++db) t.v[db] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(v0 + (size_t)db * 16 * PAGE));
   };
   auto multiply = [&](DecodeTile<D>& t, int c) {
     const int t0 = lo_al + c * CHUNK;
