@@ -107,10 +107,12 @@ def test_silu_mul(ops, dtype, inter):
         close(ops.act_mul(ops.SplitSum(parts), out_dtype=dtype, block=16), want, 1e-6 if dtype == F32 else 5e-3, "partial sums")
 
 
-# (rows, width of x, outputs): few rows run one fused kernel whose waves split K and meet in LDS; many
-# rows the tile kernels with the activation in their epilogue; 17-64 rows, few tiles, a K that is no
-# multiple of 64, or float32 run the product and the activation as two kernels. All must agree.
+# (rows, width of x, outputs): up to 64 rows run one fused kernel whose waves split K and meet in LDS
+# (K up to 2048 for up to 16 rows, up to 1024 for 17 to 64); many rows the tile kernels with the
+# activation in their epilogue; more K at few rows, few tiles, a K that is no multiple of 64, or float32
+# run the product and the activation as two kernels. All must agree.
 GATED = [(1, 1024, 3072), (8, 1024, 3072), (16, 512, 64), (5, 2048, 160), (13, 4096, 48), (40, 1024, 3072), (64, 256, 64),
+         (17, 1024, 3072), (32, 768, 160), (33, 512, 48), (64, 1024, 3072), (50, 2048, 64),
          (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096)]
 
 
