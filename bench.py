@@ -11,7 +11,9 @@ request reaches the context length. One JSON line is printed, with ``value`` = d
 second, plus the prefill rate of one 2,048-token prompt, the decode step's share of the HBM
 roofline, and decode rates at batch 1 and 64.
 
-Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32).
+Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32). Beside them the
+line carries ``measured_peaks``: what this box gives a streaming read of 1 GiB and the engine's bfloat16
+product at n = 4096, and the decode step's bytes per second as a share of that read rate.
 """
 
 from __future__ import annotations
@@ -170,6 +172,33 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * steps / d, 1)
             del e
         out["points"] = points
+
+    if not args.no_points or args.prefill_only:
+        # What this box gives beside the published peaks (the same kernels as `python -m miniserve_amd roofline`).
+        from miniserve_amd.kernels import ops
+
+        def median_ms(fn, repeats=5):
+            fn()
+            torch.cuda.synchronize()
+            times = []
+            for _ in range(repeats):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                times.append(e0.elapsed_time(e1))
+            return sorted(times)[len(times) // 2]
+
+        n = 1 << 30
+        buf = torch.empty((n,), dtype=torch.uint8, device="cuda:0").random_(0, 256)
+        read = n / median_ms(lambda: ops.measure_read(buf)) / 1e6
+        del buf
+        x = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
+        w = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
+        rate = 2 * 4096**3 / median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16)) / 1e9
+        out["measured_peaks"] = {"read_GBps": round(read, 1), "gemm_bf16_4096_TFLOPs": round(rate, 1),
+                                 "decode_frac_of_read": round(achieved / read, 4)}
 
     print(json.dumps(out))
     return 0
