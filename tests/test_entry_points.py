@@ -4,9 +4,12 @@ sources are all found by the build."""
 
 from __future__ import annotations
 
+import json
 import subprocess
 import sys
 from pathlib import Path
+
+import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
 
@@ -38,3 +41,22 @@ def test_build_finds_every_source():
             "gemm_f32.hip", "sampling.hip"} <= names
     assert [s.name for s in build.cpp_sources()] == ["block_core.cpp"]
     assert "-packed-fp32-ops" in build.HIP_FLAGS, "packed float32 instructions stay off"
+
+
+@pytest.mark.gpu
+def test_bench_line_on_a_tiny_shape():
+    """The benchmark's one JSON line with a tiny preset: every key of the contract, the flat config of
+    at most 20 keys, the prefill and roofline records, the batch 1 and 64 points."""
+    p = run(ROOT / "bench.py", "--preset", "tinyE", "--batch", "2", "--context", "512", "--steps", "4", "--warmup", "2",
+            "--prefill-tokens", "128")
+    assert p.returncode == 0, p.stderr[-2000:]
+    line = json.loads(p.stdout.strip().splitlines()[-1])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "prefill", "points"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 4 and line["warmup"] == 2 and line["value"] > 0
+    assert len(line["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in line["config"].values())
+    assert line["config"]["layers"] == line["config"]["layers_full"] == 3
+    assert set(line["roofline"]) == {"bound", "achieved", "peak", "unit", "frac"} and line["roofline"]["peak"] == 8000.0
+    assert line["prefill"]["tokens"] == 128 and line["prefill"]["value"] > 0
+    assert set(line["points"]) == {"decode_b1", "decode_b64"}
