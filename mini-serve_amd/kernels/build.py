@@ -123,9 +123,12 @@ def build_kernels(force: bool = False) -> Path:
         _run_parallel([[hipcc, *HIP_FLAGS, "-c", str(s), "-o", str(o)] for s, o in zip(srcs, objs)], "kernels")
         tmp = work / name
         _run_parallel([[hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]], "link")
-        for old in out_dir.glob("libmsamd_kernels_*.so"):
-            old.unlink(missing_ok=True)
+        # The new file takes its place in one step, and only builds of other sources are cleared away:
+        # another process that builds the same sources at the same time never finds the name missing.
         os.replace(tmp, out_dir / name)
+        for old in out_dir.glob("libmsamd_kernels_*.so"):
+            if old.name != name:
+                old.unlink(missing_ok=True)
     finally:
         shutil.rmtree(work, ignore_errors=True)
     _say("kernels built")
@@ -145,9 +148,10 @@ def build_core(force: bool = False) -> Path:
     srcs = cpp_sources()
     tmp = out_dir / f".{name}.{os.getpid()}"
     _run_parallel([[cxx, *CXX_FLAGS, "-shared", "-o", str(tmp), *map(str, srcs)]], "block core")
-    for old in out_dir.glob("libmsamd_core_*.so"):
-        old.unlink(missing_ok=True)
     os.replace(tmp, out_dir / name)
+    for old in out_dir.glob("libmsamd_core_*.so"):
+        if old.name != name:
+            old.unlink(missing_ok=True)
     return out_dir / name
 
 
