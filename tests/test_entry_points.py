@@ -60,3 +60,13 @@ def test_bench_line_on_a_tiny_shape():
     assert set(line["roofline"]) == {"bound", "achieved", "peak", "unit", "frac"} and line["roofline"]["peak"] == 8000.0
     assert line["prefill"]["tokens"] == 128 and line["prefill"]["value"] > 0
     assert set(line["points"]) == {"decode_b1", "decode_b64"}
+
+
+@pytest.mark.gpu
+def test_roofline_reports_measured_rates():
+    p = run("-m", "miniserve_amd", "roofline", "--mib", "64", "--repeats", "3")
+    assert p.returncode == 0, p.stderr[-2000:]
+    report = json.loads(p.stdout.strip().splitlines()[-1])
+    assert report["read_GBps"] > 100 and report["copy_GBps"] > 100
+    assert set(report["gemm_bf16_TFLOPs"]) == {"4096", "8192"} and all(v > 10 for v in report["gemm_bf16_TFLOPs"].values())
+    assert report["published"] == {"hbm_GBps": 8000.0, "bf16_TFLOPs": 2500.0}
