@@ -1,9 +1,8 @@
-from .allocator import BlockAllocator, OutOfBlocks
 from .manager import CacheGroup, CacheLayout, CacheManager, RequestCache, StateGroup
 from .state import OutOfStateSlots, StateSlots
-from .table import NO_BLOCK, BlockTable, pack_tables
+from .pages import NO_PAGE, OutOfBlocks, PageAllocator, PageTable, pack_tables
 
 __all__ = [
-    "BlockAllocator", "OutOfBlocks", "CacheGroup", "CacheLayout", "CacheManager", "RequestCache",
-    "StateGroup", "OutOfStateSlots", "StateSlots", "NO_BLOCK", "BlockTable", "pack_tables",
+    "PageAllocator", "OutOfBlocks", "CacheGroup", "CacheLayout", "CacheManager", "RequestCache",
+    "StateGroup", "OutOfStateSlots", "StateSlots", "NO_PAGE", "PageTable", "pack_tables",
 ]

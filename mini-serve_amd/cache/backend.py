@@ -19,9 +19,9 @@ def backend_name(name: str | None = None) -> str:
 
 def allocator_class(name: str | None = None):
     if backend_name(name) == "cpp":
-        from .native import NativeBlockAllocator
+        from .native import NativePageAllocator
 
-        return NativeBlockAllocator
-    from .allocator import BlockAllocator
+        return NativePageAllocator
+    from .pages import PageAllocator
 
-    return BlockAllocator
+    return PageAllocator

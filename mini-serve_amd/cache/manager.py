@@ -18,7 +18,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
-from .allocator import BlockAllocator, OutOfBlocks
+from .pages import OutOfBlocks, PageAllocator
 from .state import StateSlots
 
 
@@ -88,7 +88,7 @@ class CacheManager:
         pages_per_group: list[int],
         num_state_slots: int,
         max_step_tokens: int | None = None,
-        allocator_class=BlockAllocator,
+        allocator_class=PageAllocator,
     ):
         if len(pages_per_group) != len(layout.groups):
             raise ValueError("one page count per group is needed")
@@ -112,7 +112,7 @@ class CacheManager:
         return [a.num_free for a in self.allocators]
 
     def total_pages(self) -> list[int]:
-        return [a.num_blocks for a in self.allocators]
+        return [a.num_pages for a in self.allocators]
 
     def peak_pages(self, total_tokens: int, step_tokens: int | None = None) -> list[int]:
         """Most pages per group a request holds at any time on its way to ``total_tokens``, fed in
@@ -126,9 +126,10 @@ class CacheManager:
             out.append(full)
         return out
 
-    def fits_alone(self, total_tokens: int) -> bool:
-        """Whether a request of ``total_tokens`` could run with the whole pool to itself."""
-        return all(p <= t for p, t in zip(self.peak_pages(total_tokens), self.total_pages()))
+    def fits_alone(self, total_tokens: int, step_tokens: int | None = None) -> bool:
+        """Whether a request of ``total_tokens``, fed in steps of at most ``step_tokens``, could run with
+        the whole pool to itself."""
+        return all(p <= t for p, t in zip(self.peak_pages(total_tokens, step_tokens), self.total_pages()))
 
     # ------------------------------------------------------------------ request life
 
@@ -141,19 +142,19 @@ class CacheManager:
 
     def pages_needed(self, rc: RequestCache, n: int) -> list[int]:
         """Pages each group must hand out to append ``n`` tokens to ``rc`` now."""
-        return [t.blocks_needed(n) for t in rc.tables]
+        return [t.pages_needed(n) for t in rc.tables]
 
-    def outstanding(self, rc: RequestCache, total_tokens: int) -> list[int]:
+    def outstanding(self, rc: RequestCache, total_tokens: int, step_tokens: int | None = None) -> list[int]:
         """Pages per group ``rc`` may still draw (net of what it gives back) until it holds
-        ``total_tokens`` tokens."""
-        peak = self.peak_pages(total_tokens)
+        ``total_tokens`` tokens, fed in steps of at most ``step_tokens``."""
+        peak = self.peak_pages(total_tokens, step_tokens)
         out = []
         for g, t, p in zip(self.layout.groups, rc.tables, peak):
             held = t.num_held
             if g.window:
                 out.append(max(0, p - held))
             else:
-                out.append(max(0, p - t.num_blocks))
+                out.append(max(0, p - t.num_entries))
         return out
 
     def can_extend(self, rc: RequestCache, n: int) -> bool:
@@ -168,7 +169,7 @@ class CacheManager:
             if k > a.num_free:
                 raise OutOfBlocks(f"group {g}: need {k} free pages, {a.num_free} free")
         for t in rc.tables:
-            t.append_tokens(n)
+            t.append(n)
         rc.num_tokens += n
 
     def advance(self, rc: RequestCache) -> int:
@@ -198,7 +199,7 @@ class CacheManager:
 
     @property
     def idle(self) -> bool:
-        return all(a.num_free == a.num_blocks for a in self.allocators) and (
+        return all(a.num_free == a.num_pages for a in self.allocators) and (
             self.state_slots.num_free == self.state_slots.num_slots
         )
 

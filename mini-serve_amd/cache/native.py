@@ -1,4 +1,4 @@
-"""The C++ block core behind the same interface as the Python allocator and table. Built from
+"""The C++ block core behind the same interface as the Python allocator and table (``cache/pages.py``). Built from
 ``csrc/block_core.cpp`` on first use; raises the same exception types as the Python classes, so
 callers and tests cannot tell the backends apart (miniserve/cache/backend.py:46-94)."""
 
@@ -10,8 +10,7 @@ from collections.abc import Iterable
 import numpy as np
 
 from ..kernels import build
-from .allocator import OutOfBlocks
-from .table import NO_BLOCK
+from .pages import NO_PAGE, OutOfBlocks
 
 _lib = None
 _I = ctypes.c_int
@@ -56,19 +55,21 @@ def _raise(status: int, what: str):
 
 
 def _ints(values) -> np.ndarray:
-    return np.ascontiguousarray(values, dtype=np.int32)
+    if not isinstance(values, np.ndarray):
+        values = list(values)
+    return np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
 
 
-class NativeBlockAllocator:
+class NativePageAllocator:
     backend = "cpp"
 
-    def __init__(self, num_blocks: int, block_size: int):
-        if num_blocks < 1 or block_size < 1:
-            raise ValueError(f"num_blocks and block_size must be positive, got {num_blocks}, {block_size}")
+    def __init__(self, num_pages: int, page_size: int):
+        if num_pages < 1 or page_size < 1:
+            raise ValueError(f"a group needs at least one page of at least one token, got {num_pages} x {page_size}")
         self._lib = _library()
-        self._h = self._lib.msb_allocator_new(num_blocks, block_size)
-        self.num_blocks = num_blocks
-        self.block_size = block_size
+        self._h = self._lib.msb_allocator_new(num_pages, page_size)
+        self.num_pages = num_pages
+        self.page_size = page_size
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -81,50 +82,47 @@ class NativeBlockAllocator:
 
     @property
     def num_used(self) -> int:
-        return self.num_blocks - self.num_free
+        return self.num_pages - self.num_free
 
-    def can_allocate(self, n: int) -> bool:
-        return 0 <= n <= self.num_free
-
-    def refcount(self, block: int) -> int:
+    def holders_of(self, page: int) -> int:
         out = _I()
-        _raise(self._lib.msb_allocator_refcount(self._h, block, ctypes.byref(out)), f"block id {block} out of range")
+        _raise(self._lib.msb_allocator_refcount(self._h, page, ctypes.byref(out)), f"page {page} does not exist")
         return out.value
 
-    def allocate(self, n: int) -> list[int]:
+    def take(self, n: int) -> list[int]:
         if n < 0:
-            raise ValueError(f"cannot allocate {n} blocks")
+            raise ValueError(f"cannot take {n} pages")
         out = np.empty(max(n, 1), dtype=np.int32)
-        _raise(self._lib.msb_allocator_allocate(self._h, n, out.ctypes.data), f"requested {n} blocks, {self.num_free} free")
+        _raise(self._lib.msb_allocator_allocate(self._h, n, out.ctypes.data), f"{n} pages wanted, {self.num_free} free")
         return out[:n].tolist()
 
-    def incref(self, blocks: Iterable[int]) -> None:
-        a = _ints(list(blocks))
-        _raise(self._lib.msb_allocator_incref(self._h, a.ctypes.data, len(a)), f"incref of {a.tolist()}")
+    def hold(self, pages: Iterable[int]) -> None:
+        a = _ints(pages)
+        _raise(self._lib.msb_allocator_incref(self._h, a.ctypes.data, len(a)), f"cannot share pages {a.tolist()}")
 
-    def free(self, blocks: Iterable[int]) -> None:
-        a = _ints(list(blocks))
-        _raise(self._lib.msb_allocator_free(self._h, a.ctypes.data, len(a)), f"free of {a.tolist()}")
+    def give_back(self, pages: Iterable[int]) -> None:
+        a = _ints(pages)
+        _raise(self._lib.msb_allocator_free(self._h, a.ctypes.data, len(a)), f"cannot give back pages {a.tolist()}")
 
-    def new_table(self, prefix_blocks: Iterable[int] = ()):
-        return NativeBlockTable(self, list(prefix_blocks))
+    def new_table(self, shared: Iterable[int] = ()):
+        return NativePageTable(self, shared)
 
     def check_invariants(self) -> None:
-        _raise(self._lib.msb_allocator_check(self._h) and 7, "free stack disagrees with holder counts")
+        _raise(self._lib.msb_allocator_check(self._h) and 7, "the free stack and the holder counts disagree")
 
 
-class NativeBlockTable:
-    def __init__(self, allocator: NativeBlockAllocator, prefix_blocks=()):
+class NativePageTable:
+    def __init__(self, allocator: NativePageAllocator, shared=()):
         self.allocator = allocator
-        self.block_size = allocator.block_size
+        self.page_size = allocator.page_size
         self._lib = allocator._lib
-        a = _ints(list(prefix_blocks))
+        a = _ints(shared)
         st = _I()
         self._h = self._lib.msb_table_new(allocator._h, a.ctypes.data, len(a), ctypes.byref(st))
         if not self._h:
             if st.value == 9:
-                raise ValueError(f"duplicate block in prefix {a.tolist()}")
-            _raise(st.value, f"prefix {a.tolist()}")
+                raise ValueError(f"duplicate page in the shared prefix {a.tolist()}")
+            _raise(st.value, f"shared prefix {a.tolist()}")
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -136,7 +134,7 @@ class NativeBlockTable:
         return self._lib.msb_table_num_tokens(self._h)
 
     @property
-    def num_blocks(self) -> int:
+    def num_entries(self) -> int:
         return self._lib.msb_table_num_blocks(self._h)
 
     @property
@@ -145,35 +143,30 @@ class NativeBlockTable:
 
     @property
     def num_held(self) -> int:
-        return self.num_blocks - self.first_live
+        return self.num_entries - self.first_live
 
     @property
-    def capacity(self) -> int:
-        return self.num_blocks * self.block_size
-
-    @property
-    def last_block_len(self) -> int:
-        n = self.num_tokens
-        return 0 if n == 0 else n - (self.num_blocks - 1) * self.block_size
-
-    @property
-    def blocks(self) -> list[int]:
-        n = self.num_blocks
+    def entries(self) -> np.ndarray:
+        n = self.num_entries
         out = np.empty(max(n, 1), dtype=np.int32)
-        _raise(self._lib.msb_table_blocks(self._h, out.ctypes.data, n), "blocks")
-        return out[:n].tolist()
+        _raise(self._lib.msb_table_blocks(self._h, out.ctypes.data, n), "entries")
+        return out[:n]
 
-    def blocks_needed(self, n: int) -> int:
+    @property
+    def pages(self) -> list[int]:
+        return self.entries.tolist()
+
+    def pages_needed(self, n: int) -> int:
         if n < 0:
             raise ValueError(f"cannot append {n} tokens")
         return self._lib.msb_table_blocks_needed(self._h, n)
 
-    def append_tokens(self, n: int) -> list[int]:
-        k = self.blocks_needed(n)
+    def append(self, n: int) -> list[int]:
+        k = self.pages_needed(n)
         out = np.empty(max(k, 1), dtype=np.int32)
         got = _I()
         _raise(self._lib.msb_table_append(self._h, n, out.ctypes.data, len(out), ctypes.byref(got)),
-               f"requested {k} blocks, {self.allocator.num_free} free")
+               f"{k} pages wanted, {self.allocator.num_free} free")
         return out[: got.value].tolist()
 
     def slot(self, pos: int) -> int:
@@ -203,15 +196,15 @@ class NativeBlockTable:
         _raise(self._lib.msb_table_release(self._h), "release")
 
 
-def pack_native(tables, out: np.ndarray, pad_rows: int, pad_block: int) -> int:
+def pack_native(tables, out: np.ndarray, pad_rows: int, pad_page: int) -> int:
     rows, width = out.shape
     handles = (ctypes.c_void_p * max(len(tables), 1))(*[t._h for t in tables])
     total = _I()
-    st = _library().msb_pack_tables(handles, len(tables), out.ctypes.data, rows, width, pad_rows, pad_block, ctypes.byref(total))
+    st = _library().msb_pack_tables(handles, len(tables), out.ctypes.data, rows, width, pad_rows, pad_page, ctypes.byref(total))
     if st == 8:
-        raise ValueError(f"packing buffer too small: {out.shape} for {len(tables)} tables + {pad_rows} padding rows")
+        raise ValueError(f"the packing buffer is {out.shape}; {len(tables)} tables + {pad_rows} padding rows do not fit")
     _raise(st, "pack_tables")
     return total.value
 
 
-__all__ = ["NativeBlockAllocator", "NativeBlockTable", "pack_native", "NO_BLOCK"]
+__all__ = ["NativePageAllocator", "NativePageTable", "pack_native", "NO_PAGE"]

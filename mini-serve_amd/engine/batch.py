@@ -15,7 +15,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
-from ..cache.table import pack_tables
+from ..cache.pages import pack_tables
 
 
 @dataclass
@@ -93,7 +93,7 @@ class BatchBuilder:
         T = sum(lens)
         n_want = sum(len(r.want) for r in rows)
         # table rows are a multiple of 4 entries wide: kernels fetch the page ids of a key tile with one 16-byte load
-        widths = [_align(max(1, max(r.cache.tables[g].num_blocks for r in rows))) for g in range(self.num_groups)]
+        widths = [_align(max(1, max(r.cache.tables[g].num_entries for r in rows))) for g in range(self.num_groups)]
 
         seg = {}
         off = 0

@@ -8,8 +8,8 @@ token ids out; the engine never tokenizes.
 
 Overlap (one-step lag, miniserve/engine/engine.py:9-21,137-147,167-198): step t + 1 is scheduled and
 launched before the tokens of step t are read back, so the device never waits for the host's
-bookkeeping. Until then a sampled token stands in its request's output as ``PLACEHOLDER``; the next
-step takes it from the device tensor the sampler left (``StepRow.feed``). What the host learns one
+bookkeeping. Until then a sampled token is only counted by its request (``Request.in_flight``); the next
+step takes it from the device tensor the sampler left (``Request.feed``, ``StepRow.feed``). What the host learns one
 step late is a stop token: the request has then run one step too many, and the token that step
 sampled for it is dropped. Stops by length are known in advance and cost nothing. With
 ``overlap=False`` every step's tokens are read back (one copy of ``[rows]`` int32) before the next
@@ -29,7 +29,7 @@ import torch
 
 from .batch import StepRow
 from .policy import make_policy
-from .request import PLACEHOLDER, Request, RequestState, SamplingParams
+from .request import Request, RequestState, SamplingParams
 from .scheduler import Batch, Scheduler
 
 
@@ -39,7 +39,6 @@ class _Launched:
 
     batch: Batch
     sampling: list  # the requests that sample a token in this step, in row order
-    places: list  # per such request: the index in its output where the token goes
     tokens: object = None  # int32 [len(sampling)] where the sampler left them
     host: object = None  # the same on the host once ``ready`` has passed
     ready: object = None  # event after the copy to the host (None: ``host`` is valid already)
@@ -115,8 +114,8 @@ class Engine:
     # ------------------------------------------------------------------ requests
 
     def add_request(self, prompt_ids: Sequence[int], params: SamplingParams) -> Request:
-        req = Request(next(self._rids), list(prompt_ids), params)
-        req.seed = params.seed if params.seed is not None else self._seeds.randrange(2**32)
+        seed = params.seed if params.seed is not None else self._seeds.randrange(2**32)
+        req = Request(next(self._rids), prompt_ids, params, seed)
         self.scheduler.add(req)
         self.requests[req.rid] = req
         return req
@@ -148,20 +147,15 @@ class Engine:
 
     def _launch(self, batch: Batch, prev: _Launched | None) -> _Launched:
         completes = batch.completes()
-        source = {id(r): i for i, r in enumerate(prev.sampling)} if prev is not None else {}
-        rows = []
-        for r, s, n, done in zip(batch.requests, batch.starts, batch.extend_lens, completes):
-            tokens = r.token_slice(s, n)
-            # Only a request's last token can be outstanding, and only from the step before this one.
-            feed = source[id(r)] if tokens[-1] == PLACEHOLDER else None
+        rows, fed = [], False
+        for (r, start, n), done in zip(batch.rows, completes):
+            tokens, feed = r.step_tokens(start, n)  # feed: the row's last token is still in ``prev.tokens``
+            fed = fed or feed is not None
             rows.append(StepRow(r.cache, tokens, [n - 1] if done else [], feed))
-        if any(row.feed is not None for row in rows):
-            logits = self.runner.step(rows, feed_from=prev.tokens)
-        else:
-            logits = self.runner.step(rows)
+        logits = self.runner.step(rows, feed_from=prev.tokens) if fed else self.runner.step(rows)
         self.num_steps += 1
-        sampling = [r for r, done in zip(batch.requests, completes) if done]
-        launched = _Launched(batch, sampling, [len(r.output_ids) for r in sampling])
+        sampling = [r for (r, _, _), done in zip(batch.rows, completes) if done]
+        launched = _Launched(batch, sampling)
         if not sampling:
             return launched
         if self.logits_hook is not None:
@@ -174,26 +168,29 @@ class Engine:
             launched.ready.record()
         else:
             launched.host = launched.tokens
-        for r in sampling:
-            r.output_ids.append(PLACEHOLDER)
+        for i, r in enumerate(sampling):
+            r.sampled(i)
             if r.state is RequestState.PREFILL:
                 r.transition(RequestState.DECODE)
+            if r.sampled_all:
+                # Its last step is under way: the pages go back now, not at the read-back. Whoever gets them
+                # next writes them in a later step, behind this one in the stream.
+                self.runner.release(r.cache)
+                r.cache = None
         return launched
 
     def _finish(self, launched: _Launched) -> Batch:
-        """Read the step's tokens back, put them in their places, end what they end."""
+        """Read the step's tokens back, append them to their requests, end what they end."""
         if not launched.sampling:
             return launched.batch
         if launched.ready is not None:
             launched.ready.synchronize()
-        for r, at, tok in zip(launched.sampling, launched.places, launched.host.tolist()):
-            if r.is_done:  # aborted, or ended by the token before this one
+        for r, tok in zip(launched.sampling, launched.host.tolist()):
+            if r.is_done:  # aborted, or ended by the token before this one: this one ran past the end
                 self.dropped_tokens += 1
                 continue
-            r.output_ids[at] = tok
-            if at + 1 >= r.params.max_new_tokens or tok in r.params.stop_token_ids:
-                self.dropped_tokens += len(r.output_ids) - (at + 1)
-                del r.output_ids[at + 1 :]  # a placeholder of the step already under way
+            if r.read_back(tok):
+                r.forget_in_flight()  # counted as dropped when the step that sampled it is read back
                 r.transition(RequestState.FINISHED)
                 self._retire(r)
         return launched.batch

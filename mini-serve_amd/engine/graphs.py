@@ -52,7 +52,7 @@ class DecodeGraphs:
 
     def _key(self, rows):
         g = next(b for b in self.buckets if b >= len(rows))
-        need = max(max(t.num_blocks for t in r.cache.tables) for r in rows)
+        need = max(max(t.num_entries for t in r.cache.tables) for r in rows)
         w = self.MIN_WIDTH
         while w < need:
             w *= 2
@@ -138,7 +138,7 @@ class DecodeGraphs:
     def run(self, rows, starts, feed_from=None):
         """Replay the graph for these decode rows (their tables already hold the new token). Rows with
         ``feed`` take their token from the device tensor ``feed_from``."""
-        from ..cache.table import pack_tables
+        from ..cache.pages import pack_tables
 
         g, w = key = self._key(rows)
         c = self.captured.get(key)
@@ -166,7 +166,7 @@ class DecodeGraphs:
             for i, r in enumerate(rows):
                 r.cache.tables[k].tail_slots_into(1, sl[i : i + 1])
             dummy = self.runner.pool.dummy_page(k)
-            pack_tables([r.cache.tables[k] for r in rows], hv(f"table{k}").reshape(g, w), pad_rows=g - B, pad_block=dummy)
+            pack_tables([r.cache.tables[k] for r in rows], hv(f"table{k}").reshape(g, w), pad_rows=g - B, pad_page=dummy)
         if B < g:
             self._fill_padding(c, B, g, w)
         c.dev.copy_(c.host, non_blocking=True)

@@ -22,7 +22,7 @@ class ShortestJobFirst:
 
     @staticmethod
     def _remaining(r) -> int:
-        return r.params.max_new_tokens - len(r.output_ids)
+        return r.params.max_new_tokens - r.num_output
 
     def order(self, waiting):
         return sorted(waiting, key=lambda r: (r.seq_len + self._remaining(r), r.rid))

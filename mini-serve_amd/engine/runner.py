@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from ..cache.allocator import OutOfBlocks
+from ..cache.pages import OutOfBlocks
 from ..cache.manager import CacheLayout, CacheManager, RequestCache
 from ..cache.pool import KVPool
 from ..parts.model import DecoderModel

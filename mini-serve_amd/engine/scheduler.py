@@ -1,22 +1,33 @@
-"""Batch assembly: which requests run in the next step, and what happens when pages run out.
+"""Which requests run in the next step, with how many tokens each, and who gives way when pages run out.
 
-Two modes, as in the reference (miniserve/engine/scheduler.py:1-49):
+One pass builds every step, whatever the mode. The step has a token budget and the cache has, per
+layer group, a vector of free pages; both are spent in a fixed order:
 
-* ``chunked_prefill_size == 0``: prefill first. Waiting requests are admitted in order until the
-  prefill token budget is spent (the first one even if it alone exceeds it); otherwise every
-  running request decodes one token. A batch is all prefill or all decode.
-* ``chunked_prefill_size > 0``: decode first. Every decoding request gets its token; the rest of the
-  step's token budget goes to portions of prompts, first of requests part-way through their
-  prefill, then of newly admitted ones. No step runs more tokens than the budget.
+1. **Make room.** If the running requests' own next step does not fit the free pages, the newest
+   running request that holds pages gives way (never the oldest): its pages and state slot go back,
+   it keeps its tokens and returns to the front of the queue, to be prefilled again over prompt +
+   output. Repeated until the rest fits.
+2. **Decode rows**: one token for every request that is decoding.
+3. **Portions** of prompts that are part-way in (only with ``chunked_prefill_size > 0``).
+4. **Admissions**, in the policy's order, while the token budget lasts. A request is admitted only
+   if the pages it may still draw until its whole prefill and one more token are in (per group, net of
+   what windowed groups give back) fit beside what every running request may still draw. Nothing
+   is taken physically: pages are drawn step by step by the step function. The first request that
+   does not fit ends the pass: no skipping ahead.
 
-Pages. Admission takes nothing physically; it budgets: a request is admitted only if what it may
-still draw until its prefill plus one decode token is in (per cache group, net of what windowed
-groups give back) fits beside what the running requests may still draw. Admission stops at the
-first request that does not fit: no skipping ahead. When the running requests' next step does not
-fit, requests are preempted newest first (never the oldest): pages and state slot go back, the
-request keeps its output and returns to the front of the waiting queue to be prefilled again
-(prompt + output). No deadlock: a request that cannot fit the pool alone is refused at submission,
-and the oldest running request always proceeds.
+``chunked_prefill_size > 0`` (the default): the budget is that many tokens, decode rows are served
+first and count against it, prompts are cut to what is left, and one step mixes all three kinds
+of rows. ``chunked_prefill_size == 0``: prompts run whole, the budget (``max_prefill_tokens``) only
+limits how many share a step (the first is admitted even if it alone exceeds it), and a step that
+admits anything runs only the admitted prompts; decoding requests wait for the next one. These are the
+reference's two schedules (miniserve/engine/scheduler.py:1-49,156-279) and its rows step for step
+(tests/test_engine.py:141-202,286-345,355-439).
+
+No deadlock: a request that could not fit the pool alone is refused at submission, and the oldest
+request that holds pages always proceeds. A request whose every token has been sampled holds no
+pages any more (the engine gives them back at the launch of its last step, not at the read-back),
+so it never stands in anybody's way; the reference frees such requests first when pages run out
+(:281-292).
 """
 
 from __future__ import annotations
@@ -24,6 +35,8 @@ from __future__ import annotations
 import enum
 from collections import deque
 from dataclasses import dataclass, field
+
+import numpy as np
 
 from .policy import FCFS
 from .request import Request, RequestState
@@ -37,24 +50,37 @@ class Phase(enum.Enum):
 
 @dataclass
 class Batch:
-    phase: Phase
-    requests: list
-    starts: list  # tokens whose cache exists before this step, per request
-    extend_lens: list  # new tokens this step, per request
-    num_decode: int  # rows [0, num_decode) are decode rows
+    """One step's rows: ``(request, tokens already in its cache, new tokens)``, decode rows first."""
+
+    rows: list
+    num_decode: int
     preempted: list = field(default_factory=list)
 
-    def completes(self) -> list:
-        """Rows that reach the end of their sequence this step and so sample a token."""
-        return [s + n == r.seq_len for r, s, n in zip(self.requests, self.starts, self.extend_lens)]
+    @property
+    def phase(self) -> Phase:
+        if self.num_decode == len(self.rows):
+            return Phase.DECODE
+        return Phase.MIXED if self.num_decode else Phase.PREFILL
+
+    @property
+    def requests(self) -> list:
+        return [r for r, _, _ in self.rows]
+
+    @property
+    def starts(self) -> list:
+        return [s for _, s, _ in self.rows]
+
+    @property
+    def extend_lens(self) -> list:
+        return [n for _, _, n in self.rows]
 
     @property
     def num_tokens(self) -> int:
-        return sum(self.extend_lens)
+        return sum(n for _, _, n in self.rows)
 
-
-def _add(a, b):
-    return [x + y for x, y in zip(a, b)]
+    def completes(self) -> list:
+        """Per row: whether it reaches the end of its sequence in this step, and so samples a token."""
+        return [s + n == r.seq_len for r, s, n in self.rows]
 
 
 class Scheduler:
@@ -67,158 +93,135 @@ class Scheduler:
             raise ValueError("the scheduler budgets against a cache manager")
         self.max_running = max_running
         self.max_prefill_tokens = max_prefill_tokens
+        self.chunk = chunked_prefill_size
         self.cache = cache
-        self.chunked_prefill_size = chunked_prefill_size
         self.policy = policy if policy is not None else FCFS()
         self.waiting: deque = deque()
-        self.running: list = []  # admission order
+        self.running: list = []  # in admission order
         self.num_preemptions = 0
-        self.stats = dict(first_tokens=0, re_tokens=0)
+        self.stats = {"first_tokens": 0, "re_tokens": 0}  # prefill tokens of first admissions / of admissions after a preemption
 
-    # ------------------------------------------------------------------ submission
+    @property
+    def chunked_prefill_size(self) -> int:
+        return self.chunk
+
+    # ------------------------------------------------------------------ in and out
 
     def add(self, req: Request) -> None:
         if req.state is not RequestState.WAITING:
-            raise ValueError(f"request {req.rid} is {req.state.name}, expected WAITING")
-        if not self.cache.fits_alone(req.max_len):
+            raise ValueError(f"request {req.rid} is {req.state.name}; only a waiting request can be submitted")
+        # Prefilled again after a preemption it runs up to max_len - 1 tokens; whole prompts run in one step.
+        if not self.cache.fits_alone(req.max_len, self.chunk or req.max_len):
             held = [t * self.cache.page_size for t in self.cache.total_pages()]
             raise ValueError(f"request {req.rid} needs up to {req.max_len} tokens of cache, the pool holds {held}")
         self.waiting.append(req)
 
+    def retire(self, req: Request) -> None:
+        """Forget a request that has finished or was aborted, wherever it stands."""
+        if not req.is_done:
+            raise ValueError(f"request {req.rid} is {req.state.name}: only finished or aborted requests leave")
+        for queue in (self.running, self.waiting):
+            if req in queue:
+                queue.remove(req)
+                return
+
     @property
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.running) or bool(self.waiting)
 
-    def retire(self, req: Request) -> None:
-        if not req.is_done:
-            raise ValueError(f"request {req.rid} is {req.state.name}, not done")
-        if req in self.running:
-            self.running.remove(req)
-        elif req in self.waiting:
-            self.waiting.remove(req)
+    # ------------------------------------------------------------------ page vectors
 
-    # ------------------------------------------------------------------ budgets
+    def _step_of(self, req: Request) -> int:
+        """Most tokens a step carries for ``req``: what bounds the pages a windowed group holds for it."""
+        return self.chunk or req.seq_len
 
-    def _zero(self):
-        return [0] * self.cache.num_groups
-
-    @staticmethod
-    def _decodes(r: Request) -> bool:
-        return r.state is RequestState.DECODE and not r.reached_max_tokens
-
-    def _outstanding(self, reqs) -> list:
-        """Pages per group ``reqs`` may still draw before any of them finishes: the next token of
-        each decoding request, the rest of the prefill plus one token of each prefilling one."""
-        need = self._zero()
+    def _may_draw(self, reqs) -> np.ndarray:
+        """Pages per group that ``reqs`` may still take before any of them ends: the next token of each
+        decoding request, the rest of the prefill and one token of each prefilling one."""
+        need = np.zeros(self.cache.num_groups, dtype=np.int64)
         for r in reqs:
-            if self._decodes(r):
-                need = _add(need, self.cache.pages_needed(r.cache, 1))
-            elif r.state is RequestState.PREFILL:
-                need = _add(need, self.cache.outstanding(r.cache, r.seq_len + 1))
+            if r.cache is None:
+                continue  # everything sampled: it holds nothing and runs no more
+            if r.state is RequestState.PREFILL:
+                need += self.cache.outstanding(r.cache, r.seq_len + 1, self._step_of(r))
+            elif r.decodes:
+                need += self.cache.pages_needed(r.cache, 1)
         return need
 
-    def _exceeds(self, need) -> bool:
-        return any(n > f for n, f in zip(need, self.cache.free_pages()))
+    def _free(self) -> np.ndarray:
+        return np.asarray(self.cache.free_pages(), dtype=np.int64)
 
-    def _try_admit(self, req: Request, reserved) -> list | None:
-        """Acquire a cache handle for ``req`` if its whole prefill plus one token fits beside the
-        running requests and ``reserved``; returns its need, or None (nothing is left behind)."""
-        rc = self.cache.acquire()
-        need = self.cache.outstanding(rc, req.seq_len + 1)
-        spoken = _add(self._outstanding(self.running), reserved)
-        if any(n > f - s for n, f, s in zip(need, self.cache.free_pages(), spoken)):
-            self.cache.release(rc)
-            return None
-        req.cache = rc
-        return need
-
-    def _admitted(self, req: Request) -> None:
-        self.waiting.remove(req)
-        req.transition(RequestState.PREFILL)
-        self.stats["first_tokens" if req.num_preemptions == 0 else "re_tokens"] += req.seq_len
-
-    # ------------------------------------------------------------------ preemption
-
-    def _pick_victim(self, pool) -> Request:
-        candidates = [r for r in pool if r is not self.running[0]]
-        assert candidates, "a lone request does not fit in the pool"
-        return self.policy.pick_victim(candidates)
-
-    def _preempt(self, req: Request) -> None:
-        req.transition(RequestState.WAITING)
-        self.cache.release(req.cache)
-        req.cache = None
-        self.running.remove(req)
-        self.waiting.appendleft(req)
-        req.num_preemptions += 1
-        self.num_preemptions += 1
-
-    # ------------------------------------------------------------------ scheduling
+    # ------------------------------------------------------------------ the pass
 
     def schedule(self) -> Batch | None:
-        if self.chunked_prefill_size:
-            return self._schedule_chunked()
-        admitted = self._admit_whole()
-        if admitted:
-            self.running.extend(admitted)
-            return Batch(Phase.PREFILL, admitted, [0] * len(admitted), [r.seq_len for r in admitted], 0)
-        decoding = [r for r in self.running if self._decodes(r)]
-        preempted = []
-        while self._exceeds(self._outstanding(decoding)):
-            victim = self._pick_victim(decoding)
-            decoding.remove(victim)
-            self._preempt(victim)
-            preempted.append(victim)
-        if not decoding:
-            return None
-        return Batch(Phase.DECODE, decoding, [r.seq_len - 1 for r in decoding], [1] * len(decoding), len(decoding), preempted)
+        preempted = self._make_room()
+        budget = self.chunk or self.max_prefill_tokens
+        decode_rows = [(r, r.seq_len - 1, 1) for r in self.running if r.decodes]
+        rows = []
+        if self.chunk:
+            rows = list(decode_rows)
+            budget -= len(rows)
+            for r in self.running:
+                if budget <= 0:
+                    break
+                if r.state is RequestState.PREFILL:
+                    done = r.cache.num_tokens
+                    n = min(r.seq_len - done, budget)
+                    rows.append((r, done, n))
+                    budget -= n
+        admitted = self._admit(budget)
+        num_decode = len(decode_rows)
+        if self.chunk:
+            rows += admitted
+        elif admitted:
+            rows, num_decode = admitted, 0  # a step of whole prompts; decoding requests wait for the next one
+        else:
+            rows = decode_rows
+        return Batch(rows, num_decode, preempted) if rows else None
 
-    def _admit_whole(self) -> list:
-        admitted = []
-        budget = self.max_prefill_tokens
-        reserved = self._zero()
+    def _make_room(self) -> list:
+        preempted = []
+        while (self._may_draw(self.running) > self._free()).any():
+            holding = [r for r in self.running if r.cache is not None]
+            if len(holding) < 2:
+                raise RuntimeError(
+                    f"request {holding[0].rid if holding else None} does not fit the pool alone although it was admitted"
+                )
+            victim = self.policy.pick_victim(holding[1:])
+            victim.transition(RequestState.WAITING)
+            self.cache.release(victim.cache)
+            victim.cache = None
+            victim.num_preemptions += 1
+            self.num_preemptions += 1
+            self.running.remove(victim)
+            self.waiting.appendleft(victim)
+            preempted.append(victim)
+        return preempted
+
+    def _admit(self, budget: int) -> list:
+        """Admit waiting requests in the policy's order; returns their rows ``(request, 0, tokens)``."""
+        rows = []
         for req in self.policy.order(self.waiting):
-            if len(self.running) + len(admitted) >= self.max_running:
+            if len(self.running) >= self.max_running:
                 break
-            if admitted and req.seq_len > budget:
-                break  # the first request is admitted even if it alone exceeds the budget
-            need = self._try_admit(req, reserved)
-            if need is None:
+            if self.chunk:
+                if budget <= 0:
+                    break
+                n = min(req.seq_len, budget)
+            else:
+                n = req.seq_len
+                if rows and n > budget:
+                    break  # only the first prompt of a step may exceed the budget
+            handle = self.cache.acquire()
+            need = self.cache.outstanding(handle, req.seq_len + 1, self._step_of(req))
+            if (need > self._free() - self._may_draw(self.running)).any():
+                self.cache.release(handle)  # nothing stays behind a refused admission
                 break
-            reserved = _add(reserved, need)
-            self._admitted(req)
-            admitted.append(req)
-            budget -= req.seq_len
-        return admitted
-
-    def _schedule_chunked(self) -> Batch | None:
-        preempted = []
-        while self._exceeds(self._outstanding(self.running)):
-            assert len(self.running) > 1, "a lone request does not fit in the pool"
-            victim = self._pick_victim(self.running)
-            self._preempt(victim)
-            preempted.append(victim)
-        budget = self.chunked_prefill_size
-        rows = [(r, r.seq_len - 1, 1) for r in self.running if self._decodes(r)]
-        num_decode = len(rows)
-        budget -= num_decode
-        for r in self.running:
-            if r.state is RequestState.PREFILL and budget > 0:
-                start = r.cache.num_tokens
-                n = min(r.seq_len - start, budget)
-                rows.append((r, start, n))
-                budget -= n
-        for req in self.policy.order(self.waiting) if budget > 0 else ():
-            if budget <= 0 or len(self.running) >= self.max_running:
-                break
-            if self._try_admit(req, self._zero()) is None:
-                break
-            self._admitted(req)
+            req.cache = handle
+            req.transition(RequestState.PREFILL)
+            self.waiting.remove(req)
             self.running.append(req)
-            n = min(req.seq_len, budget)
+            self.stats["re_tokens" if req.num_preemptions else "first_tokens"] += req.seq_len
             rows.append((req, 0, n))
             budget -= n
-        if not rows:
-            return None
-        phase = Phase.DECODE if num_decode == len(rows) else Phase.PREFILL if num_decode == 0 else Phase.MIXED
-        return Batch(phase, [r for r, _, _ in rows], [s for _, s, _ in rows], [n for _, _, n in rows], num_decode, preempted)
+        return rows

@@ -75,20 +75,30 @@ def _writable_dir() -> Path:
 
 
 def _run_parallel(cmds: list[list[str]], what: str) -> None:
+    """Run the commands at once. Each writes to a file of its own, never to a pipe: a compiler that
+    prints more than a pipe holds would otherwise wait for a reader that only comes after its exit."""
     start = time.time()
-    procs = [(c, subprocess.Popen(c, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)) for c in cmds]
-    pending = list(procs)
+    procs = []
+    for c in cmds:
+        log = tempfile.TemporaryFile(mode="w+", prefix="msamd_log_")
+        procs.append((c, subprocess.Popen(c, stdout=log, stderr=subprocess.STDOUT, text=True), log))
     last = start
-    while pending:
-        pending = [(c, p) for c, p in pending if p.poll() is None]
-        if pending and time.time() - last > 10:
-            last = time.time()
-            _say(f"{what}: {len(pending)} of {len(procs)} still compiling ({int(last - start)} s)")
-        time.sleep(0.05)
-    for c, p in procs:
-        out = p.stdout.read()
-        if p.returncode != 0:
-            raise RuntimeError(f"build failed: {' '.join(c)}\n{out}")
+    try:
+        while any(p.poll() is None for _, p, _ in procs):
+            if time.time() - last > 10:
+                last = time.time()
+                left = sum(p.poll() is None for _, p, _ in procs)
+                _say(f"{what}: {left} of {len(procs)} still compiling ({int(last - start)} s)")
+            time.sleep(0.05)
+        for c, p, log in procs:
+            if p.returncode != 0:
+                log.seek(0)
+                raise RuntimeError(f"build failed: {' '.join(c)}\n{log.read()[-8000:]}")
+    finally:
+        for _, p, log in procs:
+            if p.poll() is None:
+                p.kill()
+            log.close()
 
 
 def kernel_library_name() -> str:

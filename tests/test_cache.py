@@ -8,21 +8,21 @@ import random
 import numpy as np
 import pytest
 
-from miniserve_amd.cache import NO_BLOCK, BlockAllocator, CacheLayout, CacheManager, OutOfBlocks, OutOfStateSlots, pack_tables
+from miniserve_amd.cache import NO_PAGE, PageAllocator, CacheLayout, CacheManager, OutOfBlocks, OutOfStateSlots, pack_tables
 from miniserve_amd.cache.backend import allocator_class
-from miniserve_amd.cache.native import NativeBlockAllocator
+from miniserve_amd.cache.native import NativePageAllocator
 from miniserve_amd.parts.base import KVNeed, StateNeed
 from miniserve_amd.parts.model import CacheSlotNeed
 
-BACKENDS = [BlockAllocator, NativeBlockAllocator]
+BACKENDS = [PageAllocator, NativePageAllocator]
 
 
 @pytest.mark.parametrize("A", BACKENDS)
 def test_allocation_order_is_part_of_the_contract(A):
     a = A(8, 4)
-    assert a.allocate(3) == [0, 1, 2] and a.allocate(2) == [3, 4]
-    a.free([1, 3])
-    assert a.allocate(1) == [3] and a.allocate(3) == [1, 5, 6]
+    assert a.take(3) == [0, 1, 2] and a.take(2) == [3, 4]
+    a.give_back([1, 3])
+    assert a.take(1) == [3] and a.take(3) == [1, 5, 6]
     assert a.num_free == 1 and a.num_used == 7
     a.check_invariants()
 
@@ -30,20 +30,20 @@ def test_allocation_order_is_part_of_the_contract(A):
 @pytest.mark.parametrize("A", BACKENDS)
 def test_allocate_is_all_or_nothing_and_free_checks_first(A):
     a = A(4, 2)
-    got = a.allocate(3)
+    got = a.take(3)
     with pytest.raises(OutOfBlocks):
-        a.allocate(2)
+        a.take(2)
     assert a.num_free == 1
     with pytest.raises(ValueError):
-        a.free([got[0], got[0]])  # one holder, two releases
+        a.give_back([got[0], got[0]])  # one holder, two releases
     with pytest.raises(IndexError):
-        a.free([got[0], 99])
-    assert a.refcount(got[0]) == 1 and a.num_free == 1  # nothing changed
-    a.incref([got[0]])
-    a.free([got[0], got[0]])
-    assert a.refcount(got[0]) == 0
+        a.give_back([got[0], 99])
+    assert a.holders_of(got[0]) == 1 and a.num_free == 1  # nothing changed
+    a.hold([got[0]])
+    a.give_back([got[0], got[0]])
+    assert a.holders_of(got[0]) == 0
     with pytest.raises(ValueError):
-        a.incref([got[0]])  # a free block
+        a.hold([got[0]])  # a free block
     with pytest.raises(ValueError):
         A(0, 4)
     a.check_invariants()
@@ -53,36 +53,36 @@ def test_allocate_is_all_or_nothing_and_free_checks_first(A):
 def test_table_vectors(A):
     a = A(8, 4)
     t = a.new_table()
-    assert t.append_tokens(5) == [0, 1] and t.blocks == [0, 1]
+    assert t.append(5) == [0, 1] and t.pages == [0, 1]
     assert [t.slot(p) for p in range(5)] == [0, 1, 2, 3, 4]
-    assert t.append_tokens(3) == [] and t.append_tokens(1) == [2] and t.slot(8) == 8
-    assert [t.blocks_needed(n) for n in (0, 3, 4, 8)] == [0, 0, 1, 2]
+    assert t.append(3) == [] and t.append(1) == [2] and t.slot(8) == 8
+    assert [t.pages_needed(n) for n in (0, 3, 4, 8)] == [0, 0, 1, 2]
     with pytest.raises(IndexError):
         t.slot(9)
     a2 = A(8, 4)
-    a2.allocate(4)
-    a2.free([1, 3])
+    a2.take(4)
+    a2.give_back([1, 3])
     t2 = a2.new_table()
-    t2.append_tokens(6)
-    assert t2.blocks == [3, 1] and t2.tail_slots(6) == [12, 13, 14, 15, 4, 5] and t2.tail_slots(2) == [4, 5]
+    t2.append(6)
+    assert t2.pages == [3, 1] and t2.tail_slots(6) == [12, 13, 14, 15, 4, 5] and t2.tail_slots(2) == [4, 5]
     t2.rewind(3)  # keeps its blocks: recomputed tokens land in the same slots
-    assert t2.num_tokens == 3 and t2.blocks == [3, 1] and t2.blocks_needed(5) == 0
+    assert t2.num_tokens == 3 and t2.pages == [3, 1] and t2.pages_needed(5) == 0
     t2.release()
-    assert t2.blocks == [] and a2.num_free == 6
+    assert t2.pages == [] and a2.num_free == 6
     with pytest.raises(OutOfBlocks):
-        A(2, 4).new_table().append_tokens(9)
+        A(2, 4).new_table().append(9)
 
 
 @pytest.mark.parametrize("A", BACKENDS)
 def test_shared_prefix(A):
     a = A(8, 4)
     first = a.new_table()
-    first.append_tokens(8)
-    second = a.new_table(first.blocks)
-    assert second.num_tokens == 8 and a.refcount(0) == 2
-    assert second.append_tokens(1) == [2]  # new tokens go to a block of its own
+    first.append(8)
+    second = a.new_table(first.pages)
+    assert second.num_tokens == 8 and a.holders_of(0) == 2
+    assert second.append(1) == [2]  # new tokens go to a block of its own
     first.release()
-    assert a.refcount(0) == 1 and a.num_free == 5
+    assert a.holders_of(0) == 1 and a.num_free == 5
     second.release()
     assert a.num_free == 8
     with pytest.raises(ValueError, match="duplicate"):
@@ -93,16 +93,16 @@ def test_shared_prefix(A):
 def test_release_before_gives_back_whole_pages_only(A):
     a = A(8, 4)
     t = a.new_table()
-    t.append_tokens(14)
+    t.append(14)
     assert t.release_before(3) == 0
-    assert t.release_before(9) == 2 and t.blocks == [NO_BLOCK, NO_BLOCK, 2, 3] and t.num_held == 2
+    assert t.release_before(9) == 2 and t.pages == [NO_PAGE, NO_PAGE, 2, 3] and t.num_held == 2
     assert a.num_free == 6 and t.release_before(9) == 0
     assert t.tail_slots(6) == [8, 9, 10, 11, 12, 13]
     with pytest.raises(IndexError):
         t.slot(7)
     with pytest.raises(IndexError):
         t.tail_slots(7)
-    assert t.append_tokens(3) == [1]  # the newest freed page comes back first
+    assert t.append(3) == [1]  # the newest freed page comes back first
     t.release()
     assert a.num_free == 8
     a.check_invariants()
@@ -114,12 +114,12 @@ def test_packing_is_the_naive_dense_layout(A):
     tables = []
     for n in (5, 0, 13):
         t = a.new_table()
-        t.append_tokens(n)
+        t.append(n)
         tables.append(t)
     tables[2].release_before(6)
     out = np.full((5, 6), 77, dtype=np.int32)
-    assert pack_tables(tables, out, pad_rows=2, pad_block=9) == 6
-    want = [[0, 1, 9, 9, 9, 9], [9] * 6, [NO_BLOCK, 3, 4, 5, 9, 9], [9] * 6, [9] * 6]
+    assert pack_tables(tables, out, pad_rows=2, pad_page=9) == 6
+    want = [[0, 1, 9, 9, 9, 9], [9] * 6, [NO_PAGE, 3, 4, 5, 9, 9], [9] * 6, [9] * 6]
     assert out.tolist() == want
     with pytest.raises(ValueError):
         pack_tables(tables, np.zeros((3, 3), dtype=np.int32))
@@ -130,7 +130,7 @@ def test_packing_is_the_naive_dense_layout(A):
 def test_backends_agree_under_random_operations():
     for seed in range(10):
         rng = random.Random(seed)
-        py, cc = BlockAllocator(24, 4), NativeBlockAllocator(24, 4)
+        py, cc = PageAllocator(24, 4), NativePageAllocator(24, 4)
         tp, tc = [], []
         for _ in range(300):
             op = rng.random()
@@ -140,12 +140,12 @@ def test_backends_agree_under_random_operations():
             if op < 0.7:
                 n = rng.randrange(0, 11)
                 try:
-                    got = tp[i].append_tokens(n)
+                    got = tp[i].append(n)
                 except OutOfBlocks:
                     with pytest.raises(OutOfBlocks):
-                        tc[i].append_tokens(n)
+                        tc[i].append(n)
                 else:
-                    assert tc[i].append_tokens(n) == got
+                    assert tc[i].append(n) == got
             elif op < 0.85:
                 pos = rng.randrange(0, tp[i].num_tokens + 1)
                 assert tp[i].release_before(pos) == tc[i].release_before(pos)
@@ -153,7 +153,7 @@ def test_backends_agree_under_random_operations():
                 tp.pop(i).release(); tc.pop(i).release()
             assert py.num_free == cc.num_free
             for a, b in zip(tp, tc):
-                assert a.blocks == b.blocks and a.num_tokens == b.num_tokens and a.num_held == b.num_held
+                assert a.pages == b.pages and a.num_tokens == b.num_tokens and a.num_held == b.num_held
             py.check_invariants(); cc.check_invariants()
 
 
@@ -243,22 +243,22 @@ def test_random_orders_of_requests_lose_no_page(backend, seed):
         elif op < 0.85:
             rc = rng.choice(live)
             n = rng.randrange(1, 10)
-            before = [(t.num_tokens, t.blocks) for t in rc.tables]
+            before = [(t.num_tokens, t.pages) for t in rc.tables]
             if m.can_extend(rc, n):
                 m.extend(rc, n)
                 m.advance(rc)
             else:
                 with pytest.raises(OutOfBlocks):
                     m.extend(rc, n)
-                assert before == [(t.num_tokens, t.blocks) for t in rc.tables]
+                assert before == [(t.num_tokens, t.pages) for t in rc.tables]
         else:
             m.release(live.pop(rng.randrange(len(live))))
         m.check_invariants()
         # every page is held by exactly one table or free
         for g, alloc in enumerate(m.allocators):
-            held = [b for rc in live for b in rc.tables[g].blocks if b != NO_BLOCK]
-            assert len(held) == len(set(held)) == alloc.num_blocks - alloc.num_free
-            assert all(alloc.refcount(b) == 1 for b in held)
+            held = [b for rc in live for b in rc.tables[g].pages if b != NO_PAGE]
+            assert len(held) == len(set(held)) == alloc.num_pages - alloc.num_free
+            assert all(alloc.holders_of(b) == 1 for b in held)
         for rc in live:
             for g, t in zip(m.layout.groups, rc.tables):
                 if g.window:

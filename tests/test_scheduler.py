@@ -8,7 +8,7 @@ import random
 import pytest
 
 from miniserve_amd.engine.engine import Engine
-from miniserve_amd.engine.request import PLACEHOLDER, InvalidTransition, Request, RequestState, SamplingParams
+from miniserve_amd.engine.request import InvalidTransition, Request, RequestState, SamplingParams
 from miniserve_amd.engine.scheduler import Phase, Scheduler
 from toy_runner import ToyRunner, ToySampler, run_alone
 
@@ -29,11 +29,12 @@ def run(batch, runner):
     from miniserve_amd.engine.batch import StepRow
 
     done = batch.completes()
-    runner.step([StepRow(r.cache, r.token_slice(s, n), [n - 1] if d else [])
-                 for r, s, n, d in zip(batch.requests, batch.starts, batch.extend_lens, done)])
+    runner.step([StepRow(r.cache, r.step_tokens(s, n)[0], [n - 1] if d else [])
+                 for (r, s, n), d in zip(batch.rows, done)])
     for r, d in zip(batch.requests, done):
         if d:
-            r.output_ids.append(0)
+            r.sampled(0)
+            r.read_back(0)
             if r.state is RequestState.PREFILL:
                 r.transition(RequestState.DECODE)
 
@@ -68,11 +69,25 @@ def test_sampling_params_are_checked():
     assert SamplingParams(1).is_greedy and not SamplingParams(1, temperature=0.5).is_greedy
 
 
-def test_token_slice_spans_prompt_and_output():
+def test_step_tokens_span_prompt_and_output_and_name_what_is_in_flight():
     r = req(0, 4)
-    r.output_ids = [9, 8, 7]
-    assert r.token_slice(0, 4) == [1, 2, 3, 4] and r.token_slice(2, 4) == [3, 4, 9, 8] and r.token_slice(5, 2) == [8, 7]
-    assert r.seq_len == 7 and r.max_len == 12
+    for tok in (9, 8, 7):
+        r.sampled(0)
+        assert not r.read_back(tok)
+    assert r.prompt_ids == [1, 2, 3, 4] and r.output_ids == [9, 8, 7]
+    assert r.step_tokens(0, 4) == ([1, 2, 3, 4], None) and r.step_tokens(2, 4) == ([3, 4, 9, 8], None)
+    assert r.step_tokens(5, 2) == ([8, 7], None) and r.seq_len == 7 and r.max_len == 12
+    r.sampled(5)  # the next token lies at index 5 of the latest step's sampled tokens, not yet on the host
+    assert r.seq_len == 8 and r.num_output == 4 and r.output_ids == [9, 8, 7]
+    assert r.step_tokens(7, 1) == ([0], 5) and r.step_tokens(5, 3) == ([8, 7, 0], 5) and r.step_tokens(5, 2) == ([8, 7], None)
+    with pytest.raises(RuntimeError):
+        r.step_tokens(7, 2)
+    r.sampled(2)  # launched once more before the read-back
+    assert r.seq_len == 9 and r.read_back(6) is False and r.seq_len == 9 and r.in_flight == 1 and r.feed == 2
+    short = Request(1, [5], SamplingParams(2, stop_token_ids={3}))
+    short.sampled(0)
+    assert not short.sampled_all and short.read_back(3) and short.forget_in_flight() == 0  # the stop token ends it and is kept
+    assert short.output_ids == [3]
 
 
 # ------------------------------------------------------------------------------------------ whole prefills
@@ -170,7 +185,7 @@ def test_lone_request_is_never_preempted_and_too_large_is_refused():
     s, runner = sched(3)
     x = req(0, 4, 8)
     s.add(x)
-    while not x.should_stop():
+    while not x.sampled_all:
         batch = s.schedule()
         assert not batch.preempted
         run(batch, runner)
@@ -253,6 +268,43 @@ def test_chunked_preempts_newest_even_mid_prefill():
     runner.cache.check_invariants()
 
 
+def test_whole_prompt_above_the_budget_holds_all_its_tokens_in_a_windowed_group():
+    """Whole prompts run in one step whatever the prefill budget, so a windowed group holds the whole
+    prompt for that step: admission and the refusal at submission count it so, and the step fits."""
+    s, runner = sched(10, chunk=0, windows=(6,), max_prefill_tokens=8)
+    with pytest.raises(ValueError, match="pool holds"):
+        s.add(req(9, 40, 2))  # 11 pages in one step although the window is 6
+    a, b = req(0, 26, 3), req(1, 26, 3)  # ceil(27 / 4) = 7 pages for the prefill step, then 2-3 behind the window
+    s.add(a); s.add(b)
+    batch = s.schedule()
+    assert rows(batch) == [(0, 0, 26)] and list(s.waiting) == [b]  # b's prompt does not fit beside a's
+    run(batch, runner)
+    assert a.cache.tables[0].num_held <= 3 and runner.cache.free_pages() == [10 - a.cache.tables[0].num_held]
+    batch = s.schedule()  # now that the window has passed most of a's pages, b is let in: alone, before a decodes
+    assert rows(batch) == [(1, 0, 26)] and not batch.preempted
+    run(batch, runner)
+    assert rows(s.schedule()) == [(0, 26, 1), (1, 26, 1)]
+    runner.cache.check_invariants()
+
+
+def test_requests_whose_tokens_are_all_sampled_hold_nothing():
+    """With the read-back one step behind, a request whose last token has been sampled gives its pages
+    back at that launch. Two requests fill a pool of 4 pages; the older one still decodes and needs a
+    page for its next token when the newer one has just sampled its last: nobody is preempted."""
+    eng = toy_engine(4, 0, overlap=True)
+    a = eng.add_request([1, 2, 3, 4, 5, 6, 7], SamplingParams(6))
+    b = eng.add_request([1, 2, 3, 4, 5, 6], SamplingParams(2))
+    eng.step()  # both prompts: 2 pages each, the pool is full
+    assert eng.runner.cache.free_pages() == [0]
+    eng.step()  # first decode step: a's 8th token fits its page; b samples its last token and lets go
+    assert b.cache is None and b.in_flight == 1 and not b.is_done and eng.runner.cache.free_pages() == [2]
+    while eng.has_unfinished:
+        eng.step()
+        eng.runner.cache.check_invariants()
+    assert eng.scheduler.num_preemptions == 0 and eng.runner.cache.idle
+    assert len(a.output_ids) == 6 and len(b.output_ids) == 2
+
+
 def test_windowed_groups_let_more_requests_in():
     """With a window of 8 the windowed group never holds more than the window plus one step, so a
     long request needs far fewer pages there than its length."""
@@ -264,7 +316,7 @@ def test_windowed_groups_let_more_requests_in():
     while s.has_unfinished and (batch := s.schedule()) is not None:
         run(batch, runner)
         for r in list(batch.requests):
-            if r.should_stop() and r.state is RequestState.DECODE:
+            if r.sampled_all and r.state is RequestState.DECODE:
                 r.transition(RequestState.FINISHED)
                 runner.release(r.cache)
                 s.retire(r)
@@ -275,35 +327,39 @@ def test_windowed_groups_let_more_requests_in():
 # ------------------------------------------------------------------------------------------ the loop under load
 
 
-def toy_engine(pages, chunk, windows=(0,), max_running=8, backend="python", seed=0, overlap=True):
+def toy_engine(pages, chunk, windows=(0,), max_running=8, backend="python", seed=0, overlap=True, max_prefill_tokens=64):
     runner = ToyRunner(pages, page_size=4, windows=windows, max_running=max_running, max_step_tokens=chunk or None, backend=backend)
-    return Engine(None, max_running=max_running, max_prefill_tokens=64, runner=runner, chunked_prefill_size=chunk,
+    return Engine(None, max_running=max_running, max_prefill_tokens=max_prefill_tokens, runner=runner, chunked_prefill_size=chunk,
                   seed=seed, sampler=ToySampler(), overlap=overlap)
 
 
 @pytest.mark.parametrize("overlap", [True, False])
 @pytest.mark.parametrize("pages,chunk,windows,backend", [
     (8, 3, (0,), "python"), (16, 0, (0,), "cpp"), (64, 2048, (0,), "python"), (8, 5, (0, 6), "cpp"), (12, 7, (10,), "python"),
+    (10, 0, (0,), "python"), (10, 0, (6,), "cpp"), (10, 0, (0, 6), "python"),
 ])
 def test_load_under_page_pressure(pages, chunk, windows, backend, overlap):
     """As the reference's load test (tests/test_engine.py:562-598): random requests and arrivals, pools
     that force preemption, whole and chunked prefill, the read-back one step behind or not; every
-    output equals the request's run alone."""
+    output equals the request's run alone. The pools of 10 pages run whole prompts of up to 30 tokens
+    under a prefill budget of 8 (a prompt above the budget is admitted alone and must hold all its
+    tokens in that one step, window or not) and new tokens up to what the pool holds."""
     preemptions = 0
-    for seed in range(6):
+    for seed in range(10 if pages == 10 else 6):
         preemptions += _load(seed, pages, chunk, windows, backend, overlap)
-    if pages == 8:
+    if pages <= 10:
         assert preemptions > 0, "the small pool was meant to force preemption"
 
 
 def _load(seed, pages, chunk, windows, backend, overlap=True) -> int:
     rng = random.Random(seed)
-    eng = toy_engine(pages, chunk, windows, backend=backend, seed=seed, overlap=overlap)
+    tight = pages == 10
+    eng = toy_engine(pages, chunk, windows, backend=backend, seed=seed, overlap=overlap, max_prefill_tokens=8 if tight else 64)
     vocab = eng.runner.model.vocab_size
     submitted = []
     pending = []
     for i in range(40):
-        n, new = rng.randint(1, 12), rng.randint(1, 16)
+        n, new = (rng.randint(1, 30), rng.randint(1, 10)) if tight else (rng.randint(1, 12), rng.randint(1, 16))
         kind = rng.choice(("greedy", "hot", "nucleus"))
         sp = SamplingParams(new, stop_token_ids=frozenset({rng.randrange(vocab)}) if rng.random() < 0.3 else frozenset(),
                             temperature=0.0 if kind == "greedy" else 4.0, top_p=0.9 if kind == "nucleus" else 1.0,
@@ -358,7 +414,7 @@ def test_overlap_drops_what_runs_past_a_stop():
                 eng.runner.cache.check_invariants()
                 steps += 1
                 assert steps < 3000
-            assert eng.runner.cache.idle and all(PLACEHOLDER not in r.output_ids for r in reqs)
+            assert eng.runner.cache.idle and all(r.in_flight == 0 for r in reqs)
             outs.append([r.output_ids for r in reqs])
             if overlap:
                 dropped += eng.dropped_tokens
