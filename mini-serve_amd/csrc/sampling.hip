@@ -5,6 +5,8 @@
 // plain temperature) are searched by SPARTS blocks each, whose best candidates a second kernel
 // compares; that second kernel also does the rows with a nucleus, one block per row, whole.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
 #define SNT 1024
 
@@ -221,5 +223,47 @@ extern "C" int ms_sample_rows(const float* logits, int rows, int vocab, long lon
                                                          (Best*)scratch);
   sample_rows_kernel<<<rows, SNT, 0, st>>>(logits, vocab, row_stride, temperature, top_p, seed, counter,
                                            (const Best*)scratch, tokens);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same two kernels over a scratch buffer that lives in the library instead of in the caller's
+// allocation, for callers that cannot allocate (declared in sampling.h).
+
+static __device__ __align__(256) unsigned char sample_static_scratch[MS_SAMPLE_STATIC_MAX_ROWS * SPARTS * sizeof(Best)];
+
+#define MS_MAX_DEVICES 64
+static void* sample_static_ptr[MS_MAX_DEVICES];  // per device: where that device's copy of the array lies
+static std::mutex sample_static_mutex;
+
+// The device address of the current device's copy of the array, looked up once per device. In host
+// code the array's name is only a handle for this lookup; kernels are given the address it returns.
+static void* sample_static_scratch_ptr() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MS_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(sample_static_mutex);
+  if (sample_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(sample_static_scratch)) != hipSuccess) return nullptr;
+    sample_static_ptr[dev] = p;
+  }
+  return sample_static_ptr[dev];
+}
+
+extern "C" int ms_sample_rows_static_max_rows() { return MS_SAMPLE_STATIC_MAX_ROWS; }
+
+extern "C" int ms_sample_rows_static(const float* logits, int rows, int vocab, long long row_stride,
+                                     const float* temperature, const float* top_p, const unsigned* seed,
+                                     const int* counter, int* tokens, hipStream_t st) {
+  if (rows <= 0) return MS_OK;
+  if (rows > MS_SAMPLE_STATIC_MAX_ROWS) return MS_UNSUPPORTED;
+  if (vocab <= 0 || row_stride < vocab || logits == nullptr || tokens == nullptr) return MS_BAD_ARG;
+  if (temperature != nullptr && (seed == nullptr || counter == nullptr)) return MS_BAD_ARG;
+  Best* parts = (Best*)sample_static_scratch_ptr();
+  if (parts == nullptr) return MS_LAUNCH_FAILED;
+  // Nothing in the array has to start at zero: the first kernel writes every part of every row that the
+  // second kernel reads (rows with a nucleus are neither written nor read), whatever an earlier call left.
+  sample_parts_kernel<<<dim3(rows, SPARTS), SPT, 0, st>>>(logits, vocab, row_stride, temperature, top_p, seed, counter, parts);
+  sample_rows_kernel<<<rows, SNT, 0, st>>>(logits, vocab, row_stride, temperature, top_p, seed, counter, parts, tokens);
   return launch_status();
 }

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "ms_attention_prefill_tile_tokens": [_c_int, _c_int],
     "ms_sample_rows": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_sample_scratch_bytes": [_c_int],
+    "ms_sample_rows_static": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
+    "ms_sample_rows_static_max_rows": [],
     "ms_measure_read": [_c_void, _c_ll, _c_int, _c_void, _c_void],
     "ms_measure_copy": [_c_void, _c_void, _c_ll, _c_int, _c_void],
 }
@@ -725,6 +727,34 @@ def sample_rows(logits, temperature=None, top_p=None, seed=None, counter=None) -
     scratch = torch.empty((need,), dtype=torch.uint8, device=logits.device)
     _check(lib.ms_sample_rows(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
                               _ptr(counter), scratch.data_ptr(), out.data_ptr(), _stream()), "sample_rows")
+    return out
+
+
+def sample_rows_static(logits, out, temperature=None, top_p=None, seed=None, counter=None) -> torch.Tensor:
+    """``sample_rows`` into the caller's ``out`` (int32 ``[rows]``) without allocating anything: the
+    candidates between the two kernels lie in an array inside the library, one per GPU, instead of
+    in a scratch tensor. For callers that cannot allocate (under graph capture, say). At most
+    ``ms_sample_rows_static_max_rows()`` rows; calls that overlap on one GPU race for the array."""
+    _dev(logits, "logits", F32, 2)
+    _dev(out, "out", I32, 1)
+    rows, vocab = logits.shape
+    if out.shape[0] != rows:
+        raise ValueError("one output element per row is needed")
+    lib = library()
+    most = lib.ms_sample_rows_static_max_rows()
+    if rows > most:
+        raise ValueError(f"sample_rows_static takes at most {most} rows, got {rows}: use sample_rows")
+    if temperature is not None:
+        _dev(temperature, "temperature", F32, 1)
+        _dev(seed, "seed", I32, 1)
+        _dev(counter, "counter", I32, 1)
+        if top_p is not None:
+            _dev(top_p, "top_p", F32, 1)
+        for v in (temperature, seed, counter) + ((top_p,) if top_p is not None else ()):
+            if v.shape[0] != rows:
+                raise ValueError("one sampling parameter per row is needed")
+    _check(lib.ms_sample_rows_static(logits.data_ptr(), rows, vocab, vocab, _ptr(temperature), _ptr(top_p), _ptr(seed),
+                                     _ptr(counter), out.data_ptr(), _stream()), "sample_rows_static")
     return out
 
 
