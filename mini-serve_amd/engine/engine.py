@@ -92,9 +92,11 @@ class Engine:
                 decode_graph_max_bs=decode_graph_max_bs,
             )
         self.runner = runner
+        spec = getattr(getattr(runner, "model", None), "spec", None)
         self.scheduler = Scheduler(
             max_running, max_prefill_tokens, cache=runner.cache, chunked_prefill_size=chunked_prefill_size,
-            policy=make_policy(schedule_policy),
+            policy=make_policy(schedule_policy), max_step_tokens=getattr(runner, "max_step_tokens_limit", None),
+            max_position=getattr(spec, "max_position", None),
         )
         if sampler is None:
             from ..sampling.sampler import Sampler

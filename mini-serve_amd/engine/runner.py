@@ -17,6 +17,8 @@ from ..cache.pool import KVPool
 from ..parts.model import DecoderModel
 from .batch import BatchBuilder, StepRow
 
+MAX_STEP_TOKENS = 65535  # what one launch of the kernels takes (``kernels.ops.MAX_STEP_TOKENS``)
+
 DEFAULT_PAGE_SIZE = 16
 
 
@@ -68,6 +70,7 @@ class ModelRunner:
             from .graphs import DecodeGraphs
 
             self.graphs = DecodeGraphs(self, decode_graph_max_bs or max_running)
+        self.max_step_tokens_limit = MAX_STEP_TOKENS
         self.steps = 0
         self.graph_steps = 0
 
@@ -98,6 +101,9 @@ class ModelRunner:
         runs ``feed_from[i]`` as its last token (the host need not have read it back)."""
         if not rows:
             return None
+        total = sum(len(r.tokens) for r in rows)
+        if total > MAX_STEP_TOKENS:
+            raise ValueError(f"a step of {total} tokens: one step carries at most {MAX_STEP_TOKENS}; cut the prompt into portions")
         vocab = self.model.vocab_size
         seen = set()
         for r in rows:

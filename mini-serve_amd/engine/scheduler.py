@@ -84,9 +84,16 @@ class Batch:
 
 
 class Scheduler:
-    def __init__(self, max_running=64, max_prefill_tokens=8192, cache=None, chunked_prefill_size=0, policy=None):
+    def __init__(self, max_running=64, max_prefill_tokens=8192, cache=None, chunked_prefill_size=0, policy=None,
+                 max_step_tokens=None, max_position=None):
+        """``max_step_tokens``: most tokens the step function takes at once (None: no limit);
+        ``max_position``: longest sequence the model is meant for (None: no limit)."""
         if max_running < 1 or max_prefill_tokens < 1:
             raise ValueError("max_running and max_prefill_tokens must be positive")
+        if max_step_tokens is not None and max(chunked_prefill_size, 0 if chunked_prefill_size else max_prefill_tokens) > max_step_tokens:
+            raise ValueError(f"a step carries at most {max_step_tokens} tokens: chunked_prefill_size / max_prefill_tokens exceed it")
+        self.max_step_tokens = max_step_tokens
+        self.max_position = max_position
         if chunked_prefill_size < 0:
             raise ValueError(f"chunked_prefill_size must be >= 0, got {chunked_prefill_size}")
         if cache is None:
@@ -110,6 +117,13 @@ class Scheduler:
     def add(self, req: Request) -> None:
         if req.state is not RequestState.WAITING:
             raise ValueError(f"request {req.rid} is {req.state.name}; only a waiting request can be submitted")
+        if self.max_position is not None and req.max_len > self.max_position:
+            # the reference's server refuses the same (miniserve/server/__main__.py:29-33)
+            raise ValueError(f"request {req.rid}: prompt + max_new_tokens = {req.max_len} tokens exceed the model's "
+                             f"max_position_embeddings = {self.max_position}")
+        if not self.chunk and self.max_step_tokens is not None and req.max_len - 1 > self.max_step_tokens:
+            raise ValueError(f"request {req.rid}: a sequence of up to {req.max_len - 1} tokens cannot run whole, one step carries "
+                             f"at most {self.max_step_tokens}: use chunked prefill")
         # Prefilled again after a preemption it runs up to max_len - 1 tokens; whole prompts run in one step.
         if not self.cache.fits_alone(req.max_len, self.chunk or req.max_len):
             held = [t * self.cache.page_size for t in self.cache.total_pages()]

@@ -303,6 +303,7 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
 # ------------------------------------------------------------------------------------- matrix products
 
 SMALL_M = 64  # rows up to which the split-K weight-streaming kernel runs
+MAX_STEP_TOKENS = 65535  # rows one launch of the matrix and elementwise kernels takes (a grid dimension)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None,

@@ -16,6 +16,8 @@ reference). ``qk_norm_eps=None`` switches the per-head norms off; ``position`` m
 
 from __future__ import annotations
 
+import warnings
+
 import torch
 
 from ..config.spec import PartSpec
@@ -37,6 +39,17 @@ class GQAttention(Mixer):
         self.window = int(spec.get("window") or 0)
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} query heads are no multiple of {self.kv_heads} KV heads")
+        # What the attention kernels refuse is refused here, when the model is built, not in its first step.
+        if self.head_dim % 16 or not 16 <= self.head_dim <= 256:
+            raise ValueError(f"head_dim {self.head_dim} is not supported: the attention kernels take multiples of 16 from 16 to 256")
+        if not self.scale > 0:
+            raise ValueError(f"the attention scale must be positive, not {self.scale}")
+        if rt is not None and rt.dtype == torch.bfloat16 and not (
+                self.head_dim in (64, 128) and self.heads // self.kv_heads <= 16):
+            warnings.warn(
+                f"attention with head_dim {self.head_dim} and {self.heads // self.kv_heads} query heads per KV head runs the "
+                "generic kernel in bfloat16 (one wave per token and head): the matrix-core kernels take head sizes 64 and 128 "
+                "with up to 16 query heads per KV head", stacklevel=2)
         pos = spec.get("position") or PartSpec("none")
         self.position = part_class("position", pos)(pos, rt)
         self.qkv = self.o = self.q_norm = self.k_norm = None

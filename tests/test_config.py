@@ -133,3 +133,23 @@ def test_registering_an_architecture():
     finally:
         unregister_architecture("ToyForCausalLM")
     assert "ToyForCausalLM" not in ARCHITECTURES
+
+
+def test_head_sizes_the_kernels_refuse_are_refused_when_the_model_is_built():
+    """Not in the first step: the attention part checks its head shape when it is constructed."""
+    from miniserve_amd.config.spec import PartSpec
+    from miniserve_amd.parts.attention import GQAttention
+
+    def spec(**kw):
+        base = dict(hidden_size=64, num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25)
+        base.update(kw)
+        return PartSpec("gqa_attention", base)
+
+    GQAttention(spec(), None)
+    for bad in (24, 8, 272, 100):
+        with pytest.raises(ValueError, match="head_dim"):
+            GQAttention(spec(head_dim=bad), None)
+    with pytest.raises(ValueError, match="no multiple"):
+        GQAttention(spec(num_heads=5), None)
+    with pytest.raises(ValueError, match="scale"):
+        GQAttention(spec(scale=0.0), None)

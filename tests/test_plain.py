@@ -1,8 +1,11 @@
 """Pins of the plain implementation beside the reference's text: special cases that reduce to a
 library routine, and invariants, each chosen so that a plausible mistake fails it (a wrong sign or
 pairing in the rotation, a norm in the wrong place or with the wrong eps, a mask off by one, a wrong
-head-to-group map). The reference's own numeric tests compare with a library model on downloaded
-weights (tests/test_consistency.py:68-145) and hold no vectors that could be reused here."""
+head-to-group map), and for the wiring of a layer (which norm feeds what, the per-head norms before the
+rotation, q_norm against k_norm, pre-norm residual sums, the final norm) a one-layer special case worked
+out in complex arithmetic plus what zeroed weights must switch off. The reference's own numeric tests
+compare with a library model on downloaded weights (tests/test_consistency.py:68-145) and hold no
+vectors that could be reused here."""
 
 import numpy as np
 import pytest
@@ -233,3 +236,185 @@ def test_nucleus_keeps_the_smallest_set_reaching_top_p():
     assert {P.sample(logits, 1.0, s, 0, top_p=0.96) for s in range(600)} == {0, 1, 2, 3}
     tie = np.log(np.array([0.25, 0.25, 0.25, 0.25]))
     assert {P.sample(tie, 1.0, s, 0, top_p=0.3) for s in range(300)} == {0, 1}  # ties stay in index order
+
+
+# ------------------------------------------------------------------------------------------ wiring of a layer
+#
+# What the part tests above cannot see: which norm feeds which product, where the per-head norms sit
+# relative to the rotation, which of q_norm / k_norm scales which side, where the residual sums and
+# the final norm sit. The library model the reference's own tests compare with is not used here (an
+# installed package's model code is no source for this build), so the wiring is pinned by a special
+# case worked out independently, in complex arithmetic, and by what must follow from zeroed weights.
+
+
+def _wiring_config(hidden, layers=1, heads=1, kv_heads=1, inter=8, vocab=None, theta=50.0, eps=1e-6):
+    return {"architectures": ["Qwen3ForCausalLM"], "hidden_size": hidden, "intermediate_size": inter,
+            "vocab_size": vocab or hidden, "num_hidden_layers": layers, "num_attention_heads": heads,
+            "num_key_value_heads": kv_heads, "head_dim": hidden // heads, "rms_norm_eps": eps, "rope_theta": theta,
+            "tie_word_embeddings": False, "max_position_embeddings": 64}
+
+
+def _random_weights(cfg, seed):
+    r = np.random.default_rng(seed)
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    w = {"model.embed_tokens.weight": r.standard_normal((V, H)), "lm_head.weight": r.standard_normal((V, H)) * 0.3,
+         "model.norm.weight": r.uniform(0.5, 1.5, H)}
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        w[p + "input_layernorm.weight"] = r.uniform(0.5, 1.5, H)
+        w[p + "post_attention_layernorm.weight"] = r.uniform(0.5, 1.5, H)
+        w[p + "self_attn.q_proj.weight"] = r.standard_normal((Hq * D, H)) * 0.4
+        w[p + "self_attn.k_proj.weight"] = r.standard_normal((Hkv * D, H)) * 0.4
+        w[p + "self_attn.v_proj.weight"] = r.standard_normal((Hkv * D, H)) * 0.4
+        w[p + "self_attn.o_proj.weight"] = r.standard_normal((H, Hq * D)) * 0.4
+        w[p + "self_attn.q_norm.weight"] = r.uniform(0.3, 1.7, D)
+        w[p + "self_attn.k_norm.weight"] = r.uniform(0.3, 1.7, D)
+        w[p + "mlp.gate_proj.weight"] = r.standard_normal((I, H)) * 0.4
+        w[p + "mlp.up_proj.weight"] = r.standard_normal((I, H)) * 0.4
+        w[p + "mlp.down_proj.weight"] = r.standard_normal((H, I)) * 0.4
+    return w
+
+
+def test_one_layer_with_identity_projections_in_closed_form():
+    """One layer, one head of the model's width, q/k/v/o projections the identity, no feed-forward
+    output, head the identity: the logits are ``norm_f(e_t + sum_s softmax_s(score_ts) x_s)`` with
+    ``x = norm_in(e)``. Pairs (j, j + D/2) are complex numbers ``z_j``; the per-head norms scale them
+    componentwise *before* the turn by ``exp(i pos theta_j)``, so the score of query t and key s is
+    ``Re sum_j a_tj conj(b_sj) exp(i (t - s) theta_j) / sqrt(D)`` with ``a = wq * rmsnorm(x_t)``,
+    ``b = wk * rmsnorm(x_s)``. Swapping q_norm and k_norm, norming after the turn, a missing or doubled
+    norm, post-norm instead of pre-norm or a wrong scale all change the result (the weights differ
+    between the two halves of a pair and between q and k)."""
+    D, T, eps, theta = 8, 6, 1e-6, 50.0
+    cfg = _wiring_config(D, theta=theta, eps=eps)
+    w = _random_weights(cfg, 5)
+    p = "model.layers.0."
+    eye = np.eye(D)
+    for n in ("q", "k", "v", "o"):
+        w[p + f"self_attn.{n}_proj.weight"] = eye
+    w[p + "mlp.down_proj.weight"] = np.zeros_like(w[p + "mlp.down_proj.weight"])
+    w["lm_head.weight"] = eye
+    ids = [3, 1, 4, 1, 5, 2]
+    got = P.logits(cfg, w, ids)
+
+    def unit(v):  # rmsnorm without a weight
+        return v / np.sqrt((v * v).mean(-1, keepdims=True) + eps)
+
+    e = w["model.embed_tokens.weight"][ids]
+    x = unit(e) * w[p + "input_layernorm.weight"]
+    a = unit(x) * w[p + "self_attn.q_norm.weight"]
+    b = unit(x) * w[p + "self_attn.k_norm.weight"]
+    half = D // 2
+    az, bz = a[:, :half] + 1j * a[:, half:], b[:, :half] + 1j * b[:, half:]
+    freq = theta ** (-np.arange(half) * 2.0 / D)
+    want = np.empty((T, D))
+    for t in range(T):
+        s = np.arange(t + 1)
+        turn = np.exp(1j * (t - s)[:, None] * freq[None, :])
+        score = (az[t][None, :] * np.conj(bz[s]) * turn).sum(-1).real / np.sqrt(D)
+        prob = np.exp(score - score.max())
+        prob /= prob.sum()
+        h = e[t] + prob @ x[s]
+        want[t] = unit(h) * w["model.norm.weight"]
+    assert np.abs(got - want).max() < 1e-5  # float32 angles in the plain implementation
+    # the pins bite: swapped per-head norm weights give other logits
+    w2 = dict(w)
+    w2[p + "self_attn.q_norm.weight"], w2[p + "self_attn.k_norm.weight"] = w[p + "self_attn.k_norm.weight"], w[p + "self_attn.q_norm.weight"]
+    assert np.abs(P.logits(cfg, w2, ids) - want).max() > 1e-3
+
+
+def test_zeroed_weights_say_which_norm_feeds_what():
+    cfg = _wiring_config(12, layers=3, heads=3, kv_heads=1, inter=10, vocab=17)
+    w = _random_weights(cfg, 6)
+    ids = [5, 16, 0, 3, 9, 9, 2]
+    base = P.logits(cfg, w, ids)
+
+    # (1) without the mixer's input nothing moves between positions: every position's logits are those of
+    # its token alone. If the other norm fed the attention, or the attention read the raw stream, they would mix.
+    w1 = dict(w)
+    for i in range(3):
+        w1[f"model.layers.{i}.input_layernorm.weight"] = np.zeros(12)
+    alone = np.stack([P.logits(cfg, w1, [t])[0] for t in ids])
+    assert np.abs(P.logits(cfg, w1, ids) - alone).max() < 1e-12 and np.abs(base - alone).max() > 1e-2
+
+    # (2) without the feed-forward's input, its weights do not matter; the attention's still do
+    w2 = dict(w)
+    for i in range(3):
+        w2[f"model.layers.{i}.post_attention_layernorm.weight"] = np.zeros(12)
+    ref = P.logits(cfg, w2, ids)
+    w2b = dict(w2)
+    for i in range(3):
+        for n in ("gate", "up", "down"):
+            w2b[f"model.layers.{i}.mlp.{n}_proj.weight"] = w2[f"model.layers.{i}.mlp.{n}_proj.weight"] * -3.0 + 1.0
+    assert np.abs(P.logits(cfg, w2b, ids) - ref).max() < 1e-12
+    w2c = dict(w2)
+    w2c["model.layers.1.self_attn.o_proj.weight"] = w2["model.layers.1.self_attn.o_proj.weight"] * 2.0
+    assert np.abs(P.logits(cfg, w2c, ids) - ref).max() > 1e-3
+
+    # (3) pre-norm: the stream itself is never normalised. With every o_proj and down_proj zero the logits
+    # are the head over the final norm of the bare embedding.
+    w3 = dict(w)
+    for i in range(3):
+        w3[f"model.layers.{i}.self_attn.o_proj.weight"] = np.zeros((12, 12))
+        w3[f"model.layers.{i}.mlp.down_proj.weight"] = np.zeros((12, 10))
+    e = w["model.embed_tokens.weight"][ids]
+    bare = e / np.sqrt((e * e).mean(-1, keepdims=True) + 1e-6) * w["model.norm.weight"] @ w["lm_head.weight"].T
+    assert np.abs(P.logits(cfg, w3, ids) - bare).max() < 1e-12
+
+    # (4) the final norm's weight multiplies what the head reads: logits are linear in it, and zero with it
+    w4 = dict(w)
+    w4["model.norm.weight"] = w["model.norm.weight"] * 2.5
+    assert np.allclose(P.logits(cfg, w4, ids), 2.5 * base, rtol=1e-12)
+    w4["model.norm.weight"] = np.zeros(12)
+    assert np.abs(P.logits(cfg, w4, ids)).max() == 0
+
+    # (5) q and k are normalised per head (their projections' scale does not matter as eps -> 0), v is not
+    cfg5 = dict(cfg, rms_norm_eps=1e-30)
+    w5 = dict(w)
+    base5 = P.logits(cfg5, w, ids)
+    for n in ("q", "k"):
+        w5[f"model.layers.1.self_attn.{n}_proj.weight"] = w[f"model.layers.1.self_attn.{n}_proj.weight"] * 7.0
+    assert np.abs(P.logits(cfg5, w5, ids) - base5).max() < 1e-9
+    w5["model.layers.1.self_attn.v_proj.weight"] = w["model.layers.1.self_attn.v_proj.weight"] * 7.0
+    assert np.abs(P.logits(cfg5, w5, ids) - base5).max() > 1e-2
+
+    # (6) a layer's norms are its own: zeroing layer 1's input norm is not the same as zeroing layer 0's
+    wa, wb = dict(w), dict(w)
+    wa["model.layers.0.input_layernorm.weight"] = np.zeros(12)
+    wb["model.layers.1.input_layernorm.weight"] = np.zeros(12)
+    assert np.abs(P.logits(cfg, wa, ids) - P.logits(cfg, wb, ids)).max() > 1e-3
+
+
+def test_hash_in_the_reference_s_own_arithmetic():
+    """The noise hash once more, in the arithmetic the reference writes it in: int64 tensors holding
+    32-bit values, products masked back to 32 bits (miniserve/engine/sampler.py:29-46); and undone by
+    the inverse steps (a multiplication by an odd constant and ``x ^= x >> 16`` are both invertible on
+    32 bits), which only works out if every shift, constant and mask is the one meant."""
+    mask, mul, golden = 0xFFFFFFFF, 0x45D9F3B, 0x9E3779B9
+
+    def mix_t(x):
+        x = ((x >> 16) ^ x) * mul & mask
+        x = ((x >> 16) ^ x) * mul & mask
+        return (x >> 16) ^ x
+
+    xs = torch.tensor([0, 1, 2, 0x7FFFFFFF, 0x80000000, 0xFFFFFFFF, 123456789, 0xDEADBEEF], dtype=torch.int64)
+    assert mix_t(xs).tolist() == [P.mix32(int(x)) for x in xs]
+    seeds, counters, vocab = torch.tensor([123, 0xFFFFFFFF], dtype=torch.int64), torch.tensor([45, 7], dtype=torch.int64), 3000
+    key = mix_t(seeds ^ mix_t(counters))
+    v = torch.arange(vocab, dtype=torch.int64) * golden
+    h = mix_t((key[:, None] + v[None, :]) & mask)
+    u = ((h >> 8).to(torch.float64) + 0.5) * (1.0 / (1 << 24))
+    for row, (s, c) in enumerate(((123, 45), (0xFFFFFFFF, 7))):
+        assert np.array_equal(u[row].numpy(), P.uniform_noise(s, c, vocab))
+    inv = pow(mul, -1, 1 << 32)
+
+    def unmix(y):
+        y ^= y >> 16
+        y = y * inv & mask
+        y ^= y >> 16
+        y = y * inv & mask
+        return y ^ (y >> 16)
+
+    for x in (0, 1, 0xFFFFFFFF, 987654321, 0x80000001):
+        assert unmix(P.mix32(x)) == x
+    assert len({P.mix32(x) for x in range(5000)}) == 5000

@@ -465,3 +465,19 @@ def test_abort_at_any_time_returns_everything(overlap):
             eng.step()
         assert rs[1].state is RequestState.ABORTED and rs[0].state is RequestState.FINISHED
         assert eng.runner.cache.idle and not eng.requests
+
+
+def test_refused_at_submission_what_could_never_run():
+    runner = ToyRunner(64, page_size=4)
+    s = Scheduler(cache=runner.cache, chunked_prefill_size=0, max_step_tokens=20, max_prefill_tokens=16, max_position=40)
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        s.add(req(0, 38, 3))  # 41 tokens at most
+    s.add(req(1, 18, 3))
+    with pytest.raises(ValueError, match="chunked prefill"):
+        s.add(req(2, 22, 2))  # prefilled again after a preemption it would run 23 tokens in one step
+    chunked = Scheduler(cache=runner.cache, chunked_prefill_size=8, max_step_tokens=20, max_position=40)
+    chunked.add(req(3, 30, 2))  # portions of 8 fit any step
+    with pytest.raises(ValueError, match="at most 20"):
+        Scheduler(cache=runner.cache, chunked_prefill_size=32, max_step_tokens=20)
+    with pytest.raises(ValueError, match="at most 20"):
+        Scheduler(cache=runner.cache, chunked_prefill_size=0, max_prefill_tokens=64, max_step_tokens=20)
