@@ -5,22 +5,33 @@ bfloat16, batch 8 at a context of 4,096 tokens per request, 16-token pages.
 
 A "step" is one decode step of the engine (schedule, one pass of the model over the batch's last
 tokens, sampling on the device, one read-back of the tokens, which the engine waits for one step
-after the launch). Requests are prefilled through the
-same step function in portions of 2,048 tokens; the timed steps are the last K before every
-request reaches the context length. One JSON line is printed, with ``value`` = decoded tokens per
-second, plus the prefill rate of one 2,048-token prompt, the decode step's share of the HBM
-roofline, and decode rates at batch 1 and 64.
+after the launch). Requests are prefilled through the same step function in portions of 2,048 tokens;
+the timed steps are the last K before every request reaches the context length. Before them run at
+least W untimed decode steps and at least ``--warmup-seconds`` of them (the number is fixed before the
+prompts are made, from a floor on the step time, so that the timed steps end at the context length;
+what the GPU's clock did meanwhile is in ``sidecar``).
 
-Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32). Beside them the
-line carries ``measured_peaks``: what this box gives a streaming read of 1 GiB and the engine's bfloat16
-product at n = 4096, and the decode step's bytes per second as a share of that read rate.
+One JSON line is printed. ``value`` = decoded tokens per second of the headline point. Beside it:
+``prefill`` (one 2,048-token prompt in one step; median of five), ``roofline`` (the decode step's bytes,
+every weight once plus the live requests' cache, over its time, against the published 8 TB/s),
+``points`` (decode at batch 1 and 64 of the same shape; with ``--extra``, on by default, the Qwen3-8B
+shape's decode at batch 1 / 8 / 64 and prefill, and the Qwen3-32B shape's continuous batching of 64
+requests with 2,048-token prompts under a 512-token step budget, decode-only and mixed steps timed
+apart, each with its share of the roofline), ``measured_peaks`` (what this box gives a streaming read
+and the engine's bfloat16 product) and ``sidecar`` (device, clocks and power while the headline point
+ran, versions, commit, the engine's effective configuration).
+
+Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32).
 """
 
 from __future__ import annotations
 
 import argparse
+import gc
 import json
+import math
 import os
+import statistics
 import sys
 import time
 
@@ -29,6 +40,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+STEP_TIME_FLOOR_S = 1.0e-3  # no decode step of these shapes is faster: sizes the warm-up by time
+
+
+def say(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
 def main() -> int:
@@ -36,12 +52,14 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--warmup-seconds", type=float, default=0.3, help="decode for at least this long before the timed steps")
     ap.add_argument("--preset", default="0.6B")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the preset has (reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill measurement")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill and the extra shapes")
+    ap.add_argument("--no-extra", action="store_true", help="skip the 8B and 32B shapes")
     ap.add_argument("--no-graph", action="store_true", help="run decode steps eagerly")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="tokens of the timed prefill step")
@@ -58,34 +76,40 @@ def main() -> int:
     from miniserve_amd.engine.batch import StepRow
     from miniserve_amd.engine.engine import Engine
     from miniserve_amd.engine.request import RequestState, SamplingParams
+    from miniserve_amd.engine.runner import ModelRunner
     from miniserve_amd.loading import random_model
+    from miniserve_amd.measurement import GpuSampler, measured_region, sidecar
+    from miniserve_amd.measurement.offline import run_to_completion
 
-    cfg = preset(args.preset)
-    full_layers = cfg["num_hidden_layers"]
-    if args.layers:
-        cfg["num_hidden_layers"] = args.layers
-    model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
-    vocab = cfg["vocab_size"]
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
     gen = torch.Generator().manual_seed(0)
 
-    def say(msg):
-        print(f"[bench] {msg}", file=sys.stderr, flush=True)
-
-    def prompts(n, length):
+    def prompts(vocab, n, length):
         return [torch.randint(0, min(vocab, 150000), (length,), generator=gen).tolist() for _ in range(n)]
 
-    def decode_run(batch: int, steps: int, warmup: int):
-        """Decode ``warmup + steps`` tokens for ``batch`` requests ending at the context length;
-        returns (seconds for the timed steps, mean context over them, engine)."""
-        total = warmup + steps
+    def make(name, layers=None):
+        cfg = preset(name)
+        full = cfg["num_hidden_layers"]
+        if layers:
+            cfg["num_hidden_layers"] = layers
+        say(f"building the {name} shape ({cfg['num_hidden_layers']} of {full} layers, {args.dtype})")
+        return cfg, full, random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
+
+    def decode_run(model, cfg, batch, steps, warmup, sampler=None, describe=False):
+        """Decode ``steps`` timed tokens for ``batch`` requests ending at the context length, after the
+        warm-up; returns a dict with the rate, the step time and the step's share of the roofline."""
+        warm_steps = max(warmup, math.ceil(args.warmup_seconds / STEP_TIME_FLOOR_S))
+        total = warm_steps + steps
         # Decoding requests keep decoding while later ones are still prefilled (about two steps per
         # request at a step budget of 2,048 tokens): prompts are shortened by that much, so that the
         # longest sequence ends at the context length.
         lead = 2 * batch
         plen = args.context - total - lead
+        if plen < 1:
+            raise SystemExit(f"context {args.context} is too short for {total} decode steps")
         eng = Engine(model, max_running=batch, kv_pool_tokens=batch * (args.context + 32), chunked_prefill_size=2048,
                      decode_graph=not args.no_graph)
-        reqs = [eng.add_request(p, SamplingParams(max_new_tokens=total + lead + 8)) for p in prompts(batch, plen)]
+        reqs = [eng.add_request(p, SamplingParams(max_new_tokens=total + lead + 8)) for p in prompts(cfg["vocab_size"], batch, plen)]
         say(f"batch {batch}: prefilling {batch} x {plen} tokens")
         last = time.time()
         while not all(r.state is RequestState.DECODE for r in reqs):
@@ -93,84 +117,135 @@ def main() -> int:
             if time.time() - last > 20:
                 last = time.time()
                 say(f"  prefill: {sum(r.cache.num_tokens for r in reqs if r.cache)} tokens in the cache")
-        say(f"batch {batch}: decoding {warmup} + {steps} steps at contexts {min(r.seq_len for r in reqs)}..{max(r.seq_len for r in reqs)}")
-        for _ in range(warmup):
+        say(f"batch {batch}: decoding {warm_steps} + {steps} steps at contexts {min(r.seq_len for r in reqs)}..{max(r.seq_len for r in reqs)}")
+        torch.cuda.synchronize()
+        w0 = time.perf_counter()
+        for _ in range(warm_steps):
             eng.step()
         torch.cuda.synchronize()
+        warm_s = time.perf_counter() - w0
+        settled = sampler.settled() if sampler is not None else None
         ctx0 = sum(r.seq_len for r in reqs) / batch
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            eng.step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
+        t_mark = sampler.sample_now() if sampler is not None else time.monotonic()
+        with measured_region(f"decode b{batch}"):
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                eng.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
         assert all(r.state is RequestState.DECODE for r in reqs), "a request ended inside the timed steps"
         mean_ctx = ctx0 + (steps - 1) / 2
+        step_bytes = model.decode_read_bytes() + batch * mean_ctx * eng.runner.pool.bytes_per_token()
+        out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "mean_ctx": mean_ctx,
+               "achieved_gbs": step_bytes / (dt / steps) / 1e9, "warmup_steps": warm_steps, "warmup_s": round(warm_s, 3),
+               "clock_settled": settled, "since": t_mark, "until": sampler.sample_now() if sampler is not None else time.monotonic()}
+        if describe:
+            out["sidecar"] = sidecar(eng)
         for r in reqs:
             eng.abort(r.rid)
-        return dt, mean_ctx, eng
+        del eng
+        return out
 
+    def prefill_run(model, cfg, T, C, repeats=5):
+        """One prompt of ``T`` tokens in one step (logits at the last position), ``C`` tokens of the same
+        sequence already cached; the median of ``repeats`` timed runs after one untimed."""
+        runner = ModelRunner(model, kv_pool_tokens=4 * T + C + 64, max_running=4)
+        vocab = cfg["vocab_size"]
+        times = []
+        for i in range(repeats + 1):
+            rc = runner.acquire()
+            ids = prompts(vocab, 1, T)[0]
+            for at in range(0, C, 2048):
+                runner.step([StepRow(rc, prompts(vocab, 1, min(2048, C - at))[0], [])])
+            torch.cuda.synchronize()
+            with measured_region("prefill") if i else measured_region("prefill (untimed)"):
+                t0 = time.perf_counter()
+                runner.step([StepRow(rc, ids, [T - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+            runner.release(rc)
+        pre = statistics.median(times[1:])
+        L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
+        Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        linear = 2 * T * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I) + 2 * H * vocab
+        attn = 2 * T * (T + 2 * C) * D * Hq * L  # causal: QK^T and PV over half the square each, and over the cached keys
+        out = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
+               "frac": round((linear + attn) / pre / PEAK_FLOPS[dt_name], 4)}
+        if C:
+            out["cached"] = C
+        del runner
+        return out
+
+    def continuous_run(model, cfg, requests=64, prompt_len=2048, new_tokens=512, budget=512):
+        """The reference's offline workload for its largest model: all requests at once, prompts cut into
+        portions under a step budget and mixed with decoding requests. Decode-only and mixed steps are
+        timed apart; a mixed step's flops are its tokens' linear products (attention aside)."""
+        eng = Engine(model, max_running=requests, kv_pool_tokens=requests * (prompt_len + new_tokens + 32),
+                     chunked_prefill_size=budget, decode_graph=not args.no_graph)
+        for p in prompts(cfg["vocab_size"], requests, prompt_len):
+            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens))
+        with measured_region("continuous batching"):
+            ran = run_to_completion(eng)
+        torch.cuda.synchronize()
+        assert eng.runner.cache.idle
+        weights = model.decode_read_bytes()
+        per_tok = eng.runner.pool.bytes_per_token()
+        L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
+        Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        flops_per_token = 2 * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I)
+        out = {"tok_s": requests * new_tokens / ran["seconds"], "seconds": ran["seconds"], "preemptions": eng.scheduler.num_preemptions}
+        d, m = ran["decode"], ran["mixed"]
+        if d["steps"]:
+            ctx = prompt_len + new_tokens / 2
+            out["decode_step_ms"] = d["median_ms"]
+            out["decode_rows"] = d["mean_rows"]
+            out["decode_frac"] = (weights + d["mean_rows"] * ctx * per_tok) / (d["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        if m["steps"]:
+            out["mixed_step_ms"] = m["median_ms"]
+            out["mixed_tokens"] = m["mean_tokens"]
+            out["mixed_frac_flops"] = flops_per_token * m["mean_tokens"] / (m["median_ms"] * 1e-3) / PEAK_FLOPS[dt_name]
+            out["mixed_frac_hbm"] = weights / (m["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        del eng
+        return out
+
+    cfg, full_layers, model = make(args.preset, args.layers)
+    vocab = cfg["vocab_size"]
+    side = {}
     if args.prefill_only:
-        dt, mean_ctx, eng = 1.0, 0.0, None
+        head = {"tok_s": 0.0, "ms_per_step": 0.0, "achieved_gbs": 0.0, "mean_ctx": 0.0, "warmup_steps": 0}
     else:
-        dt, mean_ctx, eng = decode_run(args.batch, args.steps, args.warmup)
-    ms_per_step = dt / args.steps * 1e3
-    value = args.batch * args.steps / dt
-    weight_bytes = model.decode_read_bytes()
-    kv_bytes = args.batch * mean_ctx * (eng.runner.pool.bytes_per_token() if eng else 0)
-    achieved = (weight_bytes + kv_bytes) / (dt / args.steps) / 1e9
-    del eng
+        with GpuSampler() as gpu:
+            head = decode_run(model, cfg, args.batch, args.steps, args.warmup, sampler=gpu, describe=True)
+            side = head.pop("sidecar")
+            side["warmup"] = {"steps": head["warmup_steps"], "seconds": head["warmup_s"], "clock_settled": head["clock_settled"]}
+            side["gpu_during_timed_steps"] = gpu.summary(head["since"], head["until"])
+            side["gpu_during_run"] = gpu.summary()
+    achieved = head["achieved_gbs"]
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} (Qwen3-{args.preset} shape, context {args.context})",
-        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, random token ids)",
+        "value": round(head["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt_name, "data": "synthetic (random weights, random token ids)",
         "config": {
             "model": f"Qwen3-{args.preset}-shaped", "global_batch": args.batch, "seq_len": args.context,
             "parallelism": "single GPU", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
-            "page_size": 16, "decode_graph": not args.no_graph, "overlap": True,
+            "page_size": 16, "decode_graph": not args.no_graph, "overlap": True, "warmup_steps_run": head["warmup_steps"],
+            "mean_context_timed": round(head["mean_ctx"], 1),
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
 
     if not args.no_points:
-        # Prefill of one 2,048-token prompt in one step (logits at the last position).
-        from miniserve_amd.engine.runner import ModelRunner
-
-        T, C = args.prefill_tokens, args.prefill_cached
-        runner = ModelRunner(model, kv_pool_tokens=4 * T + C + 64, max_running=4)
-        times = []
-        for i in range(4):
-            rc = runner.acquire()
-            ids = prompts(1, T)[0]
-            for at in range(0, C, 2048):
-                runner.step([StepRow(rc, prompts(1, min(2048, C - at))[0], [])])
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            runner.step([StepRow(rc, ids, [T - 1])])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            runner.release(rc)
-        pre = min(times[1:])
-        L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
-        Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-        linear = 2 * T * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I) + 2 * H * vocab
-        attn = 2 * T * (T + 2 * C) * D * Hq * L  # causal: QK^T and PV over half the square each, and over the cached keys
-        flops = linear + attn
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        out["prefill"] = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
-                          "frac": round(flops / pre / peak, 4)}
-        if C:
-            out["prefill"]["cached"] = C
-        del runner
+        out["prefill"] = prefill_run(model, cfg, args.prefill_tokens, args.prefill_cached)
         points = {}
         for b, steps in ((1, 64), (64, 24)) if not args.prefill_only else ():
-            d, _, e = decode_run(b, steps, 8)
-            points[f"decode_b{b}"] = round(b * steps / d, 1)
-            del e
+            r = decode_run(model, cfg, b, steps, 8)
+            points[f"decode_b{b}"] = round(r["tok_s"], 1)
+            points[f"decode_b{b}_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
         out["points"] = points
 
     if not args.no_points or args.prefill_only:
@@ -197,9 +272,36 @@ def main() -> int:
         x = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
         w = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
         rate = 2 * 4096**3 / median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16)) / 1e9
+        del x, w
         out["measured_peaks"] = {"read_GBps": round(read, 1), "gemm_bf16_4096_TFLOPs": round(rate, 1),
                                  "decode_frac_of_read": round(achieved / read, 4)}
 
+    if not (args.no_points or args.no_extra or args.prefill_only) and args.preset == "0.6B" and not args.layers:
+        del model
+        gc.collect()
+        torch.cuda.empty_cache()
+        points = out["points"]
+        cfg8, _, m8 = make("8B")
+        for b, steps in ((1, 32), (8, 32), (64, 16)):
+            r = decode_run(m8, cfg8, b, steps, 8)
+            points[f"8B_decode_b{b}"] = round(r["tok_s"], 1)
+            points[f"8B_decode_b{b}_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
+        p8 = prefill_run(m8, cfg8, 2048, 0)
+        points["8B_prefill_2048"] = p8["value"]
+        points["8B_prefill_2048_frac"] = p8["frac"]
+        del m8
+        gc.collect()
+        torch.cuda.empty_cache()
+        cfg32, _, m32 = make("32B")
+        c = continuous_run(m32, cfg32)
+        for k, v in c.items():
+            points[f"32B_cont64_{k}"] = round(v, 4 if "frac" in k else 2)
+        del m32
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    if side:
+        out["sidecar"] = side
     print(json.dumps(out))
     return 0
 

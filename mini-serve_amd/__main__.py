@@ -2,7 +2,8 @@
 
 * ``generate``: token ids in, token ids out, through ``Engine.generate``.
 * ``stress``: the reference's offline stress run (miniserve/tools/stress.py:28-84): random-length
-  requests of random ids, a JSON report, exit 1 unless every request finished and every page is back.
+  requests of random ids, a JSON report (decode-only and mixed step times apart, the engine's effective
+  configuration read back from it, the runtime), exit 1 unless every request finished and every page is back.
 * ``random-weights``: write a model folder with random weights.
 """
 
@@ -70,19 +71,22 @@ def cmd_stress(args) -> int:
         new = rng.randint(*args.max_new_tokens)
         ids = [rng.randrange(min(vocab, 150000)) for _ in range(n)]
         reqs.append(eng.add_request(ids, SamplingParams(new, temperature=args.temperature, top_p=args.top_p)))
-    t0 = time.time()
-    steps = 0
-    while eng.has_unfinished and steps < args.max_steps:
-        eng.step()
-        steps += 1
-    dt = time.time() - t0
+    from .measurement.offline import run_to_completion
+    from .measurement.sidecar import sidecar
+
+    ran = run_to_completion(eng, args.max_steps)
+    dt = ran["seconds"]
     finished = sum(r.state.value == "finished" for r in reqs)
     tokens = sum(len(r.output_ids) for r in reqs)
     report = {
-        "requests": len(reqs), "finished": finished, "steps": steps, "output_tokens": tokens,
+        "requests": len(reqs), "finished": finished, "steps": ran["steps"], "output_tokens": tokens,
         "seconds": round(dt, 3), "tokens_per_second": round(tokens / dt, 1) if dt > 0 else None,
-        "preemptions": eng.scheduler.num_preemptions, "idle": eng.runner.cache.idle,
+        "preemptions": eng.scheduler.num_preemptions, "dropped_tokens": eng.dropped_tokens, "idle": eng.runner.cache.idle,
+        # decode-only steps apart from steps that carry portions of prompts
+        "decode_steps": ran["decode"], "mixed_steps": ran["mixed"], "prefill_steps": ran["prefill"],
+        "stats": dict(eng.scheduler.stats),
     }
+    report.update(sidecar(eng))
     print(json.dumps(report))
     return 0 if finished == len(reqs) and eng.runner.cache.idle else 1
 

@@ -24,20 +24,24 @@ from .state import StateSlots
 
 @dataclass(frozen=True)
 class CacheGroup:
-    """Cache slots with the same needs. ``window == 0``: all keys are kept."""
+    """Cache slots that keep the same planes per token over the same window (0: every token)."""
 
     index: int
-    num_kv_heads: int
-    head_dim: int
+    planes: tuple  # of parts.base.CachePlane: name, heads, width, token_minor
     window: int
     slots: tuple[int, ...]
+
+    @property
+    def elements_per_token(self) -> int:
+        return sum(p.heads * p.width for p in self.planes)
 
 
 @dataclass(frozen=True)
 class StateGroup:
+    """The fixed-size state of one cache slot: named tensors, each with a shape per request and a dtype."""
+
     slot: int
-    shape: tuple[int, ...]
-    dtype: str
+    tensors: tuple  # of parts.base.StateTensor
 
 
 @dataclass(frozen=True)
@@ -50,19 +54,22 @@ class CacheLayout:
     def from_needs(cls, needs) -> "CacheLayout":
         """``needs``: ``CacheSlotNeed`` list of a model (``DecoderModel.cache_slots()``)."""
         by_key: dict[tuple, list[int]] = {}
+        planes_of: dict[tuple, tuple] = {}
         states = []
         for n in needs:
             if n.kv is not None:
-                by_key.setdefault((n.kv.num_kv_heads, n.kv.head_dim, n.kv.window), []).append(n.slot)
+                key = (tuple((p.name, p.heads, p.width, p.token_minor) for p in n.kv.planes), n.kv.window)
+                by_key.setdefault(key, []).append(n.slot)
+                planes_of[key] = tuple(n.kv.planes)
             if n.state is not None:
-                states.append(StateGroup(n.slot, tuple(n.state.shape), n.state.dtype))
+                states.append(StateGroup(n.slot, tuple(n.state.tensors)))
         groups = tuple(
-            CacheGroup(i, key[0], key[1], key[2], tuple(slots)) for i, (key, slots) in enumerate(sorted(by_key.items()))
+            CacheGroup(i, planes_of[key], key[1], tuple(slots)) for i, (key, slots) in enumerate(sorted(by_key.items()))
         )
         return cls(groups, tuple(states), {s: g.index for g in groups for s in g.slots})
 
     def bytes_per_page(self, page_size: int, itemsize: int) -> list[int]:
-        return [2 * len(g.slots) * page_size * g.num_kv_heads * g.head_dim * itemsize for g in self.groups]
+        return [len(g.slots) * page_size * g.elements_per_token * itemsize for g in self.groups]
 
 
 class RequestCache:

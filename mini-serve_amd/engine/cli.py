@@ -1,7 +1,8 @@
 """Command-line options shared by everything that builds an ``Engine``, under the reference's
 names and meanings where it has them (miniserve/engine/cli.py:12-106). Options of the reference
-that have nothing to switch here are still accepted, so its command lines keep working, and say so
-in their help."""
+that have nothing to switch here (``--attention``, ``--disable-radix``, ``--attn-workspace-mb``,
+``--fused-ops``: the cache is always paged, prefixes are never shared, the kernels size their own
+scratch and are always the fused ones) are not offered; argparse names them in its error."""
 
 from __future__ import annotations
 
@@ -10,15 +11,11 @@ import argparse
 from ..cache.backend import BACKENDS
 from .policy import POLICIES
 
-ATTENTION_MODES = ("paged",)
-_NO_EFFECT = " (accepted for compatibility; no effect here: "
-
 
 def add_engine_args(parser: argparse.ArgumentParser) -> None:
     g = parser.add_argument_group("engine")
     g.add_argument("--max-running", type=int, default=64, help="max requests in the running batch")
     g.add_argument("--max-prefill-tokens", type=int, default=8192, help="token budget of one prefill batch")
-    g.add_argument("--attention", choices=ATTENTION_MODES, default="paged", help="cache / attention mode")
     g.add_argument("--kv-pool-tokens", type=int, default=None,
                    help="exact cache pool size in tokens (rounded down to whole pages); default: as large as GPU memory allows")
     g.add_argument("--seed", type=int, default=0, help="seeds sampling for requests that bring no seed of their own")
@@ -36,14 +33,8 @@ def add_engine_args(parser: argparse.ArgumentParser) -> None:
                    help="page bookkeeping: python (default) or cpp; also settable with MINISERVE_BLOCK_BACKEND")
     g.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     g.add_argument("--kv-mem-fraction", type=float, default=0.9, help="share of free GPU memory the cache pool may take")
-    g.add_argument("--disable-radix", action="store_true",
-                   help="no prefix cache" + _NO_EFFECT + "prefixes are never shared between requests)")
     g.add_argument("--disable-overlap", action="store_true",
                    help="read back each step's tokens before scheduling the next (default: one step later)")
-    g.add_argument("--attn-workspace-mb", type=int, default=None,
-                   help="attention scratch buffer in MiB" + _NO_EFFECT + "the attention kernels size their own scratch)")
-    g.add_argument("--fused-ops", action="store_true",
-                   help="fused operator path" + _NO_EFFECT + "the kernels are always the fused ones)")
 
 
 def engine_kwargs(args: argparse.Namespace) -> dict:

@@ -37,33 +37,43 @@ class ModelRunner:
     ):
         """``kv_pool_tokens``: exact pool size in tokens (rounded down to whole pages; an error if
         it holds no page or does not fit, never clipped; miniserve/engine/model_runner.py:99-108);
-        default: what ``kv_mem_fraction`` of the free memory holds after a reserve for activations.
+        default: ``kv_mem_fraction`` of the memory that is free beyond the measured peak of the largest step
+        (``kv_profile`` holds the figures).
         ``max_step_tokens``: most tokens one step carries (bounds what windowed groups hold)."""
         self.model = model
         self.device = model.device
         self.page_size = page_size
         self.max_running = max_running
         self.layout = CacheLayout.from_needs(model.cache_slots())
+        self.allocator_class = allocator_class
         item = torch.empty((), dtype=model.dtype).element_size()
         per_page = sum(self.layout.bytes_per_page(page_size, item))
-        max_pages = self._pages_that_fit(per_page, kv_mem_fraction, max_step_tokens or 8192)
+        step_tokens = min(max_step_tokens or 8192, MAX_STEP_TOKENS)
+        graph_rows = (decode_graph_max_bs or max_running) if decode_graph else 0
+        self.kv_profile = {"page_size": page_size, "bytes_per_page": per_page, "kv_mem_fraction": kv_mem_fraction}
         if kv_pool_tokens is not None:
             pages = kv_pool_tokens // page_size
             if pages < 1:
                 raise ValueError(f"kv_pool_tokens={kv_pool_tokens} holds no page of {page_size} tokens")
-            if max_pages is not None and pages > max_pages:
-                raise ValueError(
-                    f"kv_pool_tokens={kv_pool_tokens} needs {pages} pages of {per_page} bytes; {max_pages} fit in memory"
-                )
+            if self.device.type == "cuda":
+                free, _ = torch.cuda.mem_get_info(self.device)
+                if pages * per_page > free:
+                    raise ValueError(
+                        f"kv_pool_tokens={kv_pool_tokens} needs {pages} pages of {per_page} bytes; {free // max(per_page, 1)} fit in memory"
+                    )
         else:
-            if max_pages is None or max_pages < 1:
-                raise RuntimeError("no memory left for the cache pool")
-            pages = max_pages
+            if per_page == 0:
+                pages = 1  # no mixer keeps anything per token: the pool is a formality
+            elif self.device.type != "cuda":
+                raise RuntimeError("the default pool size is measured on the GPU: give kv_pool_tokens")
+            else:
+                self.kv_profile.update(self._profile(step_tokens, max_running, graph_rows, kv_mem_fraction, per_page))
+                pages = self.kv_profile["max_pages"]
         self.num_pages = pages
         per_group = [pages for _ in self.layout.groups]
-        kw = {} if allocator_class is None else {"allocator_class": allocator_class}
-        self.cache = CacheManager(self.layout, page_size, per_group, max_running, max_step_tokens, **kw)
+        self.cache = CacheManager(self.layout, page_size, per_group, max_running, max_step_tokens, **self._allocator_kw())
         self.pool = KVPool(self.layout, page_size, per_group, max_running, model.dtype, self.device)
+        self.kv_profile.update(num_pages=pages, kv_pool_tokens=pages * page_size, pool_bytes=self.pool.num_bytes)
         self.builder = BatchBuilder(self.device, len(self.layout.groups))
         self.graphs = None
         if decode_graph and self.device.type == "cuda":
@@ -74,14 +84,66 @@ class ModelRunner:
         self.steps = 0
         self.graph_steps = 0
 
-    def _pages_that_fit(self, per_page: int, fraction: float, step_tokens: int) -> int | None:
-        if self.device.type != "cuda" or per_page == 0:
-            return None
-        free, _ = torch.cuda.mem_get_info(self.device)
-        spec = self.model.spec
-        widest = max([spec.hidden_size] + [b.feed_forward.spec.get("intermediate_size", 0) * 3 for b in self.model.blocks])
-        reserve = step_tokens * (spec.hidden_size * 8 + widest * 4 * 2) + self.max_running * spec.vocab_size * 8
-        return max(0, int((free - reserve) * fraction) // per_page)
+    def _allocator_kw(self) -> dict:
+        return {} if self.allocator_class is None else {"allocator_class": self.allocator_class}
+
+    def _profile(self, step_tokens: int, sample_rows: int, graph_rows: int, fraction: float, per_page: int) -> dict:
+        """How many pages fit beside what a step needs, measured, not estimated (as the reference sizes
+        its pool, miniserve/engine/model_runner.py:152-203): on a probe pool just large enough, run the
+        largest step (``step_tokens`` tokens of one request) and the largest sampling call
+        (``sample_rows`` rows with a nucleus), read the allocator's peak, then a decode step of
+        ``graph_rows`` rows, whose buffers every captured graph keeps for itself. The pool gets
+        ``fraction`` of what is free beyond those."""
+        ops = self.model.rt.ops
+        rows = max(sample_rows, graph_rows, 1)
+        probe_pages = max(-(-step_tokens // self.page_size) + 1, rows)
+        per_group = [probe_pages for _ in self.layout.groups]
+        cache = CacheManager(self.layout, self.page_size, per_group, rows, step_tokens, **self._allocator_kw())
+        pool = KVPool(self.layout, self.page_size, per_group, rows, self.model.dtype, self.device)
+        builder = BatchBuilder(self.device, len(self.layout.groups))
+
+        def peak_of(fn) -> int:
+            torch.cuda.synchronize(self.device)
+            base = torch.cuda.memory_allocated(self.device)
+            torch.cuda.reset_peak_memory_stats(self.device)
+            fn()
+            torch.cuda.synchronize(self.device)
+            return torch.cuda.max_memory_allocated(self.device) - base
+
+        def run(step_rows):
+            starts = [r.cache.num_tokens for r in step_rows]
+            for r in step_rows:
+                cache.extend(r.cache, len(r.tokens))
+            self.model.forward(builder.build(step_rows, starts), pool)
+
+        def biggest_step():
+            rc = cache.acquire()
+            run([StepRow(rc, [0] * step_tokens, [step_tokens - 1])])
+            cache.release(rc)
+            logits = torch.zeros((sample_rows, self.model.vocab_size), dtype=torch.float32, device=self.device)
+            ones = torch.ones((sample_rows,), dtype=torch.float32, device=self.device)
+            ints = torch.arange(sample_rows, dtype=torch.int32, device=self.device)
+            ops.sample_rows(logits, ones, ones * 0.9, ints, ints)
+
+        def decode_step():
+            handles = [cache.acquire() for _ in range(graph_rows)]
+            run([StepRow(rc, [0], [0]) for rc in handles])
+            for rc in handles:
+                cache.release(rc)
+
+        peak = peak_of(biggest_step)
+        graph_step = peak_of(decode_step) if graph_rows else 0
+        del pool, cache, builder
+        torch.cuda.empty_cache()
+        free, total = torch.cuda.mem_get_info(self.device)
+        # Graphs of different table widths are captured as they are needed and each keeps its step's buffers.
+        graph_reserve = 4 * graph_step
+        max_pages = int(fraction * (free - peak - graph_reserve)) // per_page
+        if max_pages < 1:
+            raise RuntimeError(f"no memory left for the cache pool: {free} bytes free, a step peaks at {peak}")
+        return {"profile_tokens": step_tokens, "profile_sample_rows": sample_rows, "peak_activation_bytes": peak,
+                "decode_step_bytes": graph_step, "graph_reserve_bytes": graph_reserve, "free_bytes": free,
+                "total_bytes": total, "max_pages": max_pages}
 
     # ------------------------------------------------------------------ request handles
 

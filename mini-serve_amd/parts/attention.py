@@ -66,8 +66,8 @@ class GQAttention(Mixer):
             p + "o_proj.weight": TensorSpec((h, hq * d)),
         }
         if spec.get("qk_norm_eps") is not None:
-            out[p + "q_norm.weight"] = TensorSpec((d,))
-            out[p + "k_norm.weight"] = TensorSpec((d,))
+            out[p + "q_norm.weight"] = TensorSpec((d,), init="ones")
+            out[p + "k_norm.weight"] = TensorSpec((d,), init="ones")
         return out
 
     def bind(self, tensors) -> None:
@@ -82,7 +82,7 @@ class GQAttention(Mixer):
             self.k_norm = tensors[p + "k_norm.weight"]
 
     def kv_need(self) -> KVNeed:
-        return KVNeed(self.kv_heads, self.head_dim, self.window)
+        return KVNeed.keys_values(self.kv_heads, self.head_dim, self.window)
 
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops

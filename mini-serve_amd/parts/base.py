@@ -6,7 +6,7 @@ those. No part knows which model it is in. The kinds:
 
 * ``Norm``            ``forward(x_f32, rows=None, add=None) -> y``  (residual stream in, compute dtype out)
 * ``PositionEncoding`` ``rotation(batch) -> Rotation | None``       (what a mixer's q/k are turned by in this step)
-* ``Mixer``           ``forward(x, batch, cache, state, residual) -> pending``
+* ``Mixer``           ``forward(x, batch, cache, state, residual) -> pending`` (``state``: name -> tensor)
 * ``FeedForward``     ``forward(x, residual) -> pending``
 * ``Block``           ``forward(residual, batch, cache, state, pending) -> pending`` (where norms and sums sit)
 * ``Embedding``       ``forward(token_ids) -> residual``            (float32 ``[T, width]``)
@@ -34,28 +34,87 @@ if TYPE_CHECKING:  # pragma: no cover
 @dataclass(frozen=True)
 class TensorSpec:
     """A tensor a part expects in the checkpoint. ``kind``: ``"float"`` tensors follow the compute
-    dtype (a tensor stored in 32-bit stays 32-bit); ``"int"`` tables are kept as int32."""
+    dtype (a tensor stored in 32-bit stays 32-bit); ``"int"`` tables are kept as int32.
+
+    ``init`` says how the random-weights mode draws it: ``"normal"`` N(0, std) (matrices, embeddings),
+    ``"ones"`` a scale around one (norm weights: all one, or uniform in the range the caller gives),
+    ``"uniform"`` U(-std, std), ``"zeros"`` (a bias that starts switched off); integer tables are
+    drawn uniformly from ``[0, high)``."""
 
     shape: tuple[int, ...]
     kind: str = "float"
+    init: str = "normal"
+    high: int | None = None
+
+    def __post_init__(self):
+        if self.kind not in ("float", "int"):
+            raise ValueError(f"unknown tensor kind {self.kind!r}")
+        if self.kind == "float" and self.init not in ("normal", "ones", "uniform", "zeros"):
+            raise ValueError(f"unknown init {self.init!r}")
+        if self.kind == "int" and (self.high is None or self.high < 1):
+            raise ValueError("an integer table needs ``high``: its entries are drawn from [0, high)")
+
+
+@dataclass(frozen=True)
+class CachePlane:
+    """One thing a mixer keeps per token in the paged cache: ``heads`` vectors of ``width`` elements.
+    Within a page a plane lies ``[page_size, width]`` per head, or, ``token_minor``, ``[width,
+    page_size]`` (the tokens of one element side by side: what a product over tokens reads)."""
+
+    name: str
+    heads: int
+    width: int
+    token_minor: bool = False
 
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values a mixer keeps per token: ``window == 0`` keeps all of them, ``window > 0``
-    only the last ``window`` (older pages may be given back)."""
+    """What a mixer keeps per token, as a list of planes (keys and values of equal or different
+    widths, one latent vector, ...). ``window == 0`` keeps every token, ``window > 0`` only the last
+    ``window`` (older pages may be given back)."""
 
-    num_kv_heads: int
-    head_dim: int
+    planes: tuple[CachePlane, ...]
     window: int = 0
+
+    def __post_init__(self):
+        names = [p.name for p in self.planes]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"cache planes need distinct names, got {names}")
+
+    @classmethod
+    def keys_values(cls, num_kv_heads: int, head_dim: int, window: int = 0) -> "KVNeed":
+        """Keys ``[page_size, head_dim]`` and values ``[head_dim, page_size]`` per KV head: what the
+        attention kernels read."""
+        return cls((CachePlane("k", num_kv_heads, head_dim), CachePlane("v", num_kv_heads, head_dim, token_minor=True)), window)
+
+    @property
+    def elements_per_token(self) -> int:
+        return sum(p.heads * p.width for p in self.planes)
+
+
+@dataclass(frozen=True)
+class StateTensor:
+    """One tensor of a mixer's per-request state: shape per request and torch dtype name."""
+
+    name: str
+    shape: tuple[int, ...]
+    dtype: str = "float32"
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Per-request state of fixed size a mixer keeps (shape per request, torch dtype name)."""
+    """Per-request state of fixed size a mixer keeps: one or several named tensors."""
 
-    shape: tuple[int, ...]
-    dtype: str = "float32"
+    tensors: tuple[StateTensor, ...]
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"state tensors need distinct names, got {names}")
+
+    @classmethod
+    def single(cls, shape, dtype: str = "float32", name: str = "state") -> "StateNeed":
+        return cls((StateTensor(name, tuple(shape), dtype),))
 
 
 @dataclass(frozen=True)

@@ -20,7 +20,7 @@ class RMSNorm(Norm):
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
-        return {spec["tensor"]: TensorSpec((int(spec["width"]),))}
+        return {spec["tensor"]: TensorSpec((int(spec["width"]),), init="ones")}
 
     def bind(self, tensors) -> None:
         self.weight = tensors[self.spec["tensor"]]

@@ -3,9 +3,11 @@
 
 The reference has no such mode; its tests alone build random tensors from the expected shapes
 and save them as a checkpoint (tests/test_weights.py:26-32). Tensors are drawn in sorted name
-order from one seeded generator: matrices and embeddings from N(0, std), norm weights either all
-one or uniform in ``norm_range``. Values are rounded to bfloat16 before they are stored, so the
-float32 and the bfloat16 path start from the same numbers.
+order from one seeded generator, each by the rule its part declares (``TensorSpec.init``): ``normal``
+N(0, std) for matrices and embeddings, ``ones`` for norm weights (all one, or uniform in
+``norm_range``), ``uniform`` U(-std, std), ``zeros``; integer tables uniformly from ``[0, high)``.
+Float values are rounded to bfloat16 before they are stored, so the float32 and the bfloat16 path
+start from the same numbers.
 """
 
 from __future__ import annotations
@@ -35,23 +37,29 @@ def random_tensors(
     dtype: torch.dtype = torch.bfloat16,
     device: str | torch.device = "cpu",
 ) -> dict[str, torch.Tensor]:
-    """Name -> tensor for every tensor the model's parts declare. One-dimensional float tensors
-    are taken to be norm weights. Drawing happens on ``device`` (a GPU generator draws other
-    numbers than the CPU's; a folder written once is what fixes the values)."""
+    """Name -> tensor for every tensor the model's parts declare, each drawn by its own ``init``
+    rule. Drawing happens on ``device`` (a GPU generator draws other numbers than the CPU's; a
+    folder written once is what fixes the values)."""
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)
+    f32 = dict(dtype=torch.float32, device=device)
     out = {}
     for name, ts in sorted(expected_tensors(spec).items()):
         if ts.kind == "int":
-            raise NotImplementedError(f"{name}: no random rule for integer tables")
-        if len(ts.shape) == 1:
+            out[name] = torch.randint(0, ts.high, ts.shape, generator=gen, dtype=torch.int32, device=device)
+            continue
+        if ts.init == "ones":
             if init.norm_range is None:
-                t = torch.ones(ts.shape, dtype=torch.float32, device=device)
+                t = torch.ones(ts.shape, **f32)
             else:
                 lo, hi = init.norm_range
-                t = torch.rand(ts.shape, generator=gen, dtype=torch.float32, device=device) * (hi - lo) + lo
+                t = torch.rand(ts.shape, generator=gen, **f32) * (hi - lo) + lo
+        elif ts.init == "zeros":
+            t = torch.zeros(ts.shape, **f32)
+        elif ts.init == "uniform":
+            t = (torch.rand(ts.shape, generator=gen, **f32) * 2 - 1) * init.std
         else:
-            t = torch.randn(ts.shape, generator=gen, dtype=torch.float32, device=device) * init.std
+            t = torch.randn(ts.shape, generator=gen, **f32) * init.std
         out[name] = t.to(torch.bfloat16).to(dtype)
     return out
 

@@ -11,7 +11,7 @@ import pytest
 from miniserve_amd.cache import NO_PAGE, PageAllocator, CacheLayout, CacheManager, OutOfBlocks, OutOfStateSlots, pack_tables
 from miniserve_amd.cache.backend import allocator_class
 from miniserve_amd.cache.native import NativePageAllocator
-from miniserve_amd.parts.base import KVNeed, StateNeed
+from miniserve_amd.parts.base import CachePlane, KVNeed, StateNeed, StateTensor
 from miniserve_amd.parts.model import CacheSlotNeed
 
 BACKENDS = [PageAllocator, NativePageAllocator]
@@ -161,20 +161,51 @@ def test_backends_agree_under_random_operations():
 
 
 def layout(windows=(0, 0, 8), state=False):
-    needs = [CacheSlotNeed(i, KVNeed(2, 16, w), StateNeed((3,)) if state and i == 0 else None) for i, w in enumerate(windows)]
+    needs = [CacheSlotNeed(i, KVNeed.keys_values(2, 16, w), StateNeed.single((3,)) if state and i == 0 else None)
+             for i, w in enumerate(windows)]
     return CacheLayout.from_needs(needs)
 
 
 def test_layers_are_grouped_by_their_needs():
     lay = CacheLayout.from_needs([
-        CacheSlotNeed(0, KVNeed(2, 16, 8), None), CacheSlotNeed(1, KVNeed(2, 16, 0), None),
-        CacheSlotNeed(2, KVNeed(2, 16, 8), None), CacheSlotNeed(3, KVNeed(1, 32, 0), StateNeed((4, 2))),
-        CacheSlotNeed(4, None, StateNeed((5,))),
+        CacheSlotNeed(0, KVNeed.keys_values(2, 16, 8), None), CacheSlotNeed(1, KVNeed.keys_values(2, 16, 0), None),
+        CacheSlotNeed(2, KVNeed.keys_values(2, 16, 8), None), CacheSlotNeed(3, KVNeed.keys_values(1, 32, 0), StateNeed.single((4, 2))),
+        CacheSlotNeed(4, None, StateNeed((StateTensor("sum", (5,)), StateTensor("seen", (1,), "int32")))),
     ])
-    assert [(g.num_kv_heads, g.head_dim, g.window, g.slots) for g in lay.groups] == [
+    assert [(g.planes[0].heads, g.planes[0].width, g.window, g.slots) for g in lay.groups] == [
         (1, 32, 0, (3,)), (2, 16, 0, (1,)), (2, 16, 8, (0, 2))]
-    assert [(s.slot, s.shape) for s in lay.states] == [(3, (4, 2)), (4, (5,))]
+    assert all([p.name for p in g.planes] == ["k", "v"] and g.planes[1].token_minor and not g.planes[0].token_minor for g in lay.groups)
+    assert [(s.slot, [(t.name, t.shape, t.dtype) for t in s.tensors]) for s in lay.states] == [
+        (3, [("state", (4, 2), "float32")]), (4, [("sum", (5,), "float32"), ("seen", (1,), "int32")])]
     assert lay.bytes_per_page(16, 2) == [2 * 1 * 16 * 32 * 2, 2 * 1 * 16 * 32 * 2, 2 * 2 * 16 * 32 * 2]
+
+
+def test_the_pool_is_built_from_what_the_mixers_say_they_keep():
+    """A mixer names its per-token record as planes: keys and values of different widths, or one latent
+    vector per token, get pages of their own shape without a change to the pool; state may be several
+    tensors of different dtypes."""
+    import torch
+
+    from miniserve_amd.cache.pool import KVPool
+
+    lay = CacheLayout.from_needs([
+        CacheSlotNeed(0, KVNeed((CachePlane("k", 2, 32), CachePlane("v", 2, 16, token_minor=True)), 0), None),
+        CacheSlotNeed(1, KVNeed((CachePlane("latent", 1, 24),), 0), StateNeed((StateTensor("sum", (6,)), StateTensor("seen", (1,), "int32")))),
+        CacheSlotNeed(2, KVNeed((CachePlane("latent", 1, 24),), 0), None),
+    ])
+    assert [[p.name for p in g.planes] for g in lay.groups] == [["k", "v"], ["latent"]] and lay.groups[1].slots == (1, 2)
+    assert lay.bytes_per_page(4, 2) == [1 * 4 * (2 * 32 + 2 * 16) * 2, 2 * 4 * 24 * 2]
+    pool = KVPool(lay, 4, [5, 7], 3, torch.bfloat16, "cpu")
+    assert tuple(pool.buffers[0]["k"].shape) == (1, 6, 2, 4, 32) and tuple(pool.buffers[0]["v"].shape) == (1, 6, 2, 16, 4)
+    assert tuple(pool.buffers[1]["latent"].shape) == (2, 8, 1, 4, 24)
+    assert pool.bytes_per_token() == (96 + 2 * 24) * 2 and pool.dummy_page(1) == 7
+    state = pool.state_view(1, None)
+    assert tuple(state["sum"].shape) == (4, 6) and state["sum"].dtype == torch.float32
+    assert tuple(state["seen"].shape) == (4, 1) and state["seen"].dtype == torch.int32 and pool.state_view(0, None) is None
+    with pytest.raises(ValueError, match="distinct names"):
+        KVNeed((CachePlane("k", 1, 8), CachePlane("k", 1, 8)))
+    with pytest.raises(ValueError, match="distinct names"):
+        StateNeed(())
 
 
 @pytest.mark.parametrize("backend", ["python", "cpp"])

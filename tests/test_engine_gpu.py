@@ -198,3 +198,37 @@ def test_stress_run_finishes_and_returns_every_page(folders):
     assert res.returncode == 0, res.stdout[-1000:] + res.stderr[-2000:]
     report = json.loads(res.stdout.strip().splitlines()[-1])
     assert report["finished"] == 24 and report["idle"]
+    # decode-only and mixed steps are timed apart; the effective configuration is read back from the engine
+    assert report["decode_steps"]["steps"] > 0 and report["mixed_steps"]["steps"] > 0
+    assert report["decode_steps"]["median_ms"] > 0 and report["mixed_steps"]["mean_tokens"] > report["decode_steps"]["mean_tokens"]
+    eng = report["engine"]
+    assert eng["kv_pool_tokens"] == [640] and eng["page_size"] == 16 and eng["chunked_prefill_size"] == 64
+    assert eng["max_running"] == 8 and eng["architecture"] == "Qwen3ForCausalLM" and eng["overlap"] is True
+    assert report["runtime"]["gpu"] and report["runtime"]["torch"]
+
+
+def test_default_pool_is_sized_from_a_measured_peak(folders):
+    """Without ``kv_pool_tokens`` the pool takes a share of what is free beyond the measured peak of
+    the largest step (miniserve/engine/model_runner.py:152-203); the figures can be read back."""
+    import torch
+
+    from miniserve_amd.engine.describe import engine_description
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyD"])
+    free, _ = torch.cuda.mem_get_info()
+    eng = engine(folders["tinyD"], "bfloat16", max_running=4, chunked_prefill_size=256, kv_mem_fraction=0.02)
+    prof = eng.runner.kv_profile
+    assert prof["profile_tokens"] == 256 and prof["profile_sample_rows"] == 4
+    assert prof["peak_activation_bytes"] > 256 * cfg["hidden_size"] * 4  # at least the float32 stream of the profiled step
+    assert prof["decode_step_bytes"] > 0 and prof["graph_reserve_bytes"] == 4 * prof["decode_step_bytes"]
+    assert prof["num_pages"] == prof["max_pages"] == int(0.02 * (prof["free_bytes"] - prof["peak_activation_bytes"]
+                                                                 - prof["graph_reserve_bytes"])) // prof["bytes_per_page"]
+    assert 0.01 * free < prof["pool_bytes"] <= 0.02 * free + prof["bytes_per_page"]
+    d = engine_description(eng)
+    assert d["kv_pool_pages"] == [prof["num_pages"]] and d["kv_profile"]["max_pages"] == prof["max_pages"]
+    prompts = prompts_for(cfg, [30, 5])
+    got = eng.generate(prompts, SamplingParams(max_new_tokens=6))
+    assert [len(g) for g in got] == [6, 6] and eng.runner.cache.idle
+    with pytest.raises(ValueError, match="fit in memory"):
+        engine(folders["tinyD"], "bfloat16", kv_pool_tokens=2**40)

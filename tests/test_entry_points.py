@@ -46,9 +46,9 @@ def test_build_finds_every_source():
 @pytest.mark.gpu
 def test_bench_line_on_a_tiny_shape():
     """The benchmark's one JSON line with a tiny preset: every key of the contract, the flat config of
-    at most 20 keys, the prefill and roofline records, the batch 1 and 64 points."""
+    at most 20 keys, the prefill and roofline records, the batch 1 and 64 points, the sidecar."""
     p = run(ROOT / "bench.py", "--preset", "tinyE", "--batch", "2", "--context", "512", "--steps", "4", "--warmup", "2",
-            "--prefill-tokens", "128")
+            "--prefill-tokens", "128", "--warmup-seconds", "0.02")
     assert p.returncode == 0, p.stderr[-2000:]
     line = json.loads(p.stdout.strip().splitlines()[-1])
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
@@ -59,7 +59,12 @@ def test_bench_line_on_a_tiny_shape():
     assert line["config"]["layers"] == line["config"]["layers_full"] == 3
     assert set(line["roofline"]) == {"bound", "achieved", "peak", "unit", "frac"} and line["roofline"]["peak"] == 8000.0
     assert line["prefill"]["tokens"] == 128 and line["prefill"]["value"] > 0
-    assert set(line["points"]) == {"decode_b1", "decode_b64"}
+    assert set(line["points"]) == {"decode_b1", "decode_b1_frac", "decode_b64", "decode_b64_frac"}
+    assert line["config"]["warmup_steps_run"] == 20  # at least --warmup steps and --warmup-seconds at a millisecond a step
+    side = line["sidecar"]
+    assert side["runtime"]["torch"] and side["runtime"]["kernel_library"].startswith("libmsamd_kernels_")
+    assert side["engine"]["kv_pool_tokens"] == [2 * (512 + 32)] * 2 and side["engine"]["decode_graph"] is True
+    assert side["engine"]["chunked_prefill_size"] == 2048 and side["warmup"]["steps"] == 20
 
 
 @pytest.mark.gpu

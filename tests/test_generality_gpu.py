@@ -23,11 +23,13 @@ ROT_DIM, POS_STEP = 8, 0.5  # the toy position encoding turns pair j of the firs
 @pytest.fixture(scope="module")
 def toy():
     from miniserve_amd.config import LayerSpec, ModelSpec, PartSpec, RunEntry, register_architecture, unregister_architecture
-    from miniserve_amd.parts import FeedForward, Mixer, PositionEncoding, Rotation, StateNeed, TensorSpec, register, unregister
+    from miniserve_amd.parts import FeedForward, Mixer, PositionEncoding, Rotation, StateNeed, StateTensor, TensorSpec, register, unregister
 
     @register("mixer", "toy_decay")
     class DecayMixer(Mixer):
-        """s_t = decay * s_{t-1} + x_t per request (s starts at 0); output = s_t W^T."""
+        """s_t = decay * s_{t-1} + x_t per request (s starts at 0), n_t = tokens seen so far (this one
+        included); output = (s_t / (1 + n_t / 8) + bias) W^T. The state is two tensors of different
+        dtypes (the float32 sum and the int32 count), the bias a one-dimensional tensor that is no norm weight."""
 
         def __init__(self, spec, rt):
             super().__init__(spec, rt)
@@ -35,32 +37,38 @@ def toy():
 
         @classmethod
         def tensors(cls, spec):
-            return {"toy.weight": TensorSpec((int(spec["width"]), int(spec["width"])))}
+            w = int(spec["width"])
+            return {"toy.weight": TensorSpec((w, w)), "toy.bias": TensorSpec((w,), init="uniform")}
 
         def bind(self, tensors):
-            self.weight = tensors["toy.weight"]
+            self.weight, self.bias = tensors["toy.weight"], tensors["toy.bias"]
 
         def state_need(self):
-            return StateNeed((self.width,), "float32")
+            return StateNeed((StateTensor("sum", (self.width,), "float32"), StateTensor("seen", (1,), "int32")))
 
         def forward(self, x, batch, cache, state, residual):
             xf = x.float()
+            total, seen = state["sum"], state["seen"]
             slots = batch.state_slots.long()
             if batch.is_decode:  # one token per row: no host loop, capturable in a graph
-                s = torch.where(batch.starts[:, None] == 0, torch.zeros_like(xf), state[slots]) * self.decay + xf
-                state[slots] = s
-                out = s
+                fresh = batch.starts[:, None] == 0
+                s = torch.where(fresh, torch.zeros_like(xf), total[slots]) * self.decay + xf
+                n = torch.where(fresh, torch.zeros_like(seen[slots]), seen[slots]) + 1
+                total[slots], seen[slots] = s, n
+                out = s / (1 + n.float() / 8)
             else:
                 out = torch.empty_like(xf)
                 t = 0
                 for i, (n, start) in enumerate(zip(batch.row_lens, batch.row_starts_host)):
                     slot = slots[i]
-                    s = torch.zeros(self.width, device=xf.device) if start == 0 else state[slot].clone()
+                    s = torch.zeros(self.width, device=xf.device) if start == 0 else total[slot].clone()
                     for j in range(n):
                         s = s * self.decay + xf[t + j]
-                        out[t + j] = s
-                    state[slot] = s
+                        out[t + j] = s / (1 + (start + j + 1) / 8)
+                    total[slot] = s
+                    seen[slot] = start + n
                     t += n
+            out = out + self.bias.float()
             return self.rt.ops.linear(out.to(x.dtype).contiguous(), self.weight, accumulate_into=residual, defer=True)
 
     @register("feed_forward", "toy_routed")
@@ -172,7 +180,7 @@ def plain_toy(w, ids):
     s, outs = np.zeros(H), []
     for t in range(T):
         s = DECAY * s + x[t]
-        outs.append(s)
+        outs.append(s / (1 + (t + 1) / 8) + w["l0.toy.bias"])
     h = h + np.stack(outs) @ w["l0.toy.weight"].T
     # routed feed-forward: the expert with the largest router logit, weighted by its softmax weight
     y = P.rms_norm(h, w["l0.n2.weight"], 1e-5)
@@ -228,8 +236,10 @@ def test_toy_architecture_runs_through_the_engine(toy, dtype):
     weights = random_tensors(spec, 7, Init(0.08, (0.6, 1.4)), dtype=rt.dtype, device=rt.device)
     model = DecoderModel(spec, weights, rt)
     needs = model.cache_slots()
-    assert [n.slot for n in needs] == [0, 1, 2] and needs[0].kv is None and needs[0].state.shape == (H,)
-    assert needs[1].kv.head_dim == D and needs[1].state is None
+    assert [n.slot for n in needs] == [0, 1, 2] and needs[0].kv is None
+    assert [(t.name, t.shape, t.dtype) for t in needs[0].state.tensors] == [("sum", (H,), "float32"), ("seen", (1,), "int32")]
+    assert [(p.name, p.heads, p.width) for p in needs[1].kv.planes] == [("k", KVH, D), ("v", KVH, D)] and needs[1].state is None
+    assert weights["l0.toy.bias"].float().abs().max() > 0.01, "the bias was meant to be drawn, not taken for a norm weight"
 
     runner = ModelRunner(model, kv_pool_tokens=16 * 12, max_running=4, decode_graph=True)
     assert [g.slots for g in runner.layout.groups] == [(1, 2)] and [s.slot for s in runner.layout.states] == [0]

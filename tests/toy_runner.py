@@ -31,7 +31,7 @@ def pseudo_logits(tokens, vocab) -> np.ndarray:
 
 class ToyRunner:
     def __init__(self, num_pages, page_size=4, vocab=50, windows=(0,), max_running=8, max_step_tokens=None, backend="python"):
-        needs = [CacheSlotNeed(i, KVNeed(1, 16, w), None) for i, w in enumerate(windows)]
+        needs = [CacheSlotNeed(i, KVNeed.keys_values(1, 16, w), None) for i, w in enumerate(windows)]
         self.layout = CacheLayout.from_needs(needs)
         self.cache = CacheManager(self.layout, page_size, [num_pages] * len(self.layout.groups), max_running,
                                   max_step_tokens, allocator_class=allocator_class(backend))
