@@ -428,13 +428,14 @@ __global__ __launch_bounds__(D) void attn_decode_reduce_kernel(const float* __re
 template <bool FUSED>
 static int launch_decode(const bf16* q, int q_stride, bf16* kc, bf16* vc, const int* block_table, int table_width,
                          const int* tokens, const int* token_row, const int* pos, bf16* out, float* part_o, float* part_ml,
-                         int rows, int splits, int Hq, int Hkv, int D, float scale, int window, FusedQkv fin, hipStream_t st) {
+                         int rows, int splits, int Hq, int Hkv, int D, float scale, int window, FusedQkv fin, hipStream_t st,
+                         bool reduce = true) {
   dim3 grid(rows * Hkv, splits);
 #define LAUNCH(DD)                                                                                                      \
   attn_decode_split_kernel<DD, FUSED><<<grid, 256, 0, st>>>(q, q_stride, kc, vc, block_table, table_width, tokens,      \
                                                             token_row, pos, out, part_o, part_ml, Hq, Hkv, scale,       \
                                                             window, fin);                                               \
-  if (splits > 1) attn_decode_reduce_kernel<DD><<<dim3(rows, Hq), DD, 0, st>>>(part_o, part_ml, tokens, out, Hq, splits)
+  if (splits > 1 && reduce) attn_decode_reduce_kernel<DD><<<dim3(rows, Hq), DD, 0, st>>>(part_o, part_ml, tokens, out, Hq, splits)
   if (D == 128) { LAUNCH(128); } else { LAUNCH(64); }
 #undef LAUNCH
   return launch_status();
@@ -464,11 +465,12 @@ extern "C" int ms_attention_decode_fused_bf16(const float* parts, int qkv_splits
                                               int store, void* kc, void* vc, const int* block_table, int table_width,
                                               const int* tokens, const int* token_row, const int* pos, void* out,
                                               float* part_o, float* part_ml, int rows, int splits, int Hq, int Hkv, int D,
-                                              int page_size, float scale, int window, hipStream_t st) {
+                                              int page_size, float scale, int window, int reduce, hipStream_t st) {
   if (rows <= 0) return MS_OK;
   if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || splits < 1 || splits > 65535 || window < 0 || table_width <= 0 ||
-      (splits > 1 && (!part_o || !part_ml)) || parts == nullptr || qkv_splits < 1 || qkv_split_stride % 4 ||
+      (splits > 1 && (!part_o || !part_ml)) || (splits > 1 && reduce && out == nullptr) || (splits == 1 && out == nullptr) ||
+      parts == nullptr || qkv_splits < 1 || qkv_split_stride % 4 ||
       (q_weight == nullptr) != (k_weight == nullptr))
     return MS_BAD_ARG;
   FusedQkv fin;
@@ -482,5 +484,147 @@ extern "C" int ms_attention_decode_fused_bf16(const float* parts, int qkv_splits
   fin.rope = rope;
   fin.store = store;
   return launch_decode<true>(nullptr, 0, (bf16*)kc, (bf16*)vc, block_table, table_width, tokens, token_row, pos, (bf16*)out,
-                             part_o, part_ml, rows, splits, Hq, Hkv, D, scale, window, fin, st);
+                             part_o, part_ml, rows, splits, Hq, Hkv, D, scale, window, fin, st, reduce != 0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The reduction of the splits and the output projection in one kernel, for up to 16 rows that bring one
+// token each: Y[m, n] = sum over heads h, d of out[m, h, d] W[n, h D + d], out being what the reduction
+// kernel above would have written. A block owns HB heads (a slice of K) and NW * 16 rows of W, one wave
+// per 16 rows. Its waves first ask for their weights, then merge the splits of the block's heads for every
+// row (a wave per (row, head): a lane per split finds the maximum and the weights by wave reductions;
+// then every thread sums its elements over the splits in ascending order), leave the merged rows in LDS
+// as bfloat16, and multiply. K is split over the grid by heads: block column c writes the float partial
+// sums P[c, m, n], which the reader of the residual stream adds up as it does for the other products
+// of few rows. At most 64 splits (a lane each).
+#define MERGE_MAX_SPLITS 64
+#define MERGE_MAX_HB 4
+template <int D, int NW>
+__global__ __launch_bounds__(NW * WAVE) void attn_merge_project_kernel(const float* __restrict__ part_o,
+                                                                       const float* __restrict__ part_ml,
+                                                                       const bf16* __restrict__ W, float* __restrict__ P,
+                                                                       int rows, int Hq, int splits, int HB, int N) {
+  __shared__ float fw[MERGE_MAX_HB][16][MERGE_MAX_SPLITS];            // weight of split s in row m of head j
+  __shared__ __attribute__((aligned(16))) bf16 xs[16][MERGE_MAX_HB * D + 8];  // merged rows; rows beyond `rows` are zero
+  __shared__ float4 psum[NW * WAVE];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int h0 = blockIdx.x * HB;          // first head of this block
+  const int K = Hq * D, KB = HB * D;       // columns of W; of this block
+  const int nb = (blockIdx.y * NW + wave) * 16;
+  // weights first: they come from memory, everything below from the cache
+  constexpr int STEPS = MERGE_MAX_HB * D / 64;
+  union Chunk { uint4 u; bf16x8 v; };
+  Chunk a[STEPS][2];
+  const bool row_in = nb + 16 <= N;
+  {
+    const bf16* wp = W + (size_t)min(nb + r, N - 1) * K + (size_t)h0 * D + g * 16;
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      if (u * 64 < KB) {
+        a[u][0].u = *reinterpret_cast<const uint4*>(wp + u * 64);
+        a[u][1].u = *reinterpret_cast<const uint4*>(wp + u * 64 + 8);
+      } else {
+        a[u][0].u = a[u][1].u = make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
+  for (int e = tid; e < 16 * MERGE_MAX_HB * (D / 4); e += NW * WAVE)  // rows beyond `rows` and heads beyond HB read as zero
+    *reinterpret_cast<uint2*>(&xs[e / (MERGE_MAX_HB * (D / 4))][(e % (MERGE_MAX_HB * (D / 4))) * 4]) = make_uint2(0, 0);
+  // the weights of the splits: wave w takes the (row, head) pairs w, w + NW, ...
+  for (int p = wave; p < rows * HB; p += NW) {
+    const int m = p / HB, j = p % HB;
+    const float2* ml = reinterpret_cast<const float2*>(part_ml) + ((size_t)m * Hq + h0 + j) * splits;
+    const float2 q = lane < splits ? ml[lane] : make_float2(-INFINITY, 0.f);
+    const float mx = wave_max(q.x);
+    const float f = q.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(q.x - mx);  // an empty or absent split adds nothing
+    const float total = wave_sum(q.y * f);
+    fw[j][m][lane] = f / total;
+  }
+  __syncthreads();
+  // Merged rows. An element is four consecutive d of one (row, head); there are E = rows * HB * D / 4 of
+  // them. With fewer elements than threads the splits of an element are shared out among SG threads
+  // (contiguous ranges, each summed in ascending order, the ranges then added in ascending order), so
+  // that one row's 64 splits are not one thread's 64 dependent loads.
+  const int E = rows * HB * (D / 4);
+  const int threads = NW * WAVE;
+  const int SG = E >= threads ? 1 : threads / E;
+  const int per = (splits + SG - 1) / SG;
+  for (int base = 0; base < E * SG; base += threads) {
+    const int item = base + tid;
+    const bool live = item < E * SG;
+    const int e = live ? item % E : 0, sg = live ? item / E : 0;
+    const int m = e / (HB * (D / 4)), c = e % (HB * (D / 4));
+    const int j = c / (D / 4), d = (c % (D / 4)) * 4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int s_end = min(splits, (sg + 1) * per);
+    if (live) {
+      const float* po = part_o + (((size_t)m * Hq + h0 + j) * splits) * D + d;
+      for (int s0 = sg * per; s0 < s_end; s0 += 8) {
+        float4 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const float4*>(po + (size_t)min(s0 + u, splits - 1) * D);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const float f = s0 + u < s_end ? fw[j][m][s0 + u] : 0.f;
+          acc.x += t[u].x * f; acc.y += t[u].y * f; acc.z += t[u].z * f; acc.w += t[u].w * f;
+        }
+      }
+    }
+    if (SG > 1) {  // then E * SG <= threads: one round
+      psum[tid] = acc;
+      __syncthreads();
+      if (tid < E) {
+        acc = psum[tid];
+        for (int q = 1; q < SG; ++q) {
+          const float4 t = psum[q * E + tid];
+          acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+        }
+      }
+    }
+    if (live && sg == 0) {
+      union { uint2 u; bf16 b[4]; } o;
+      o.b[0] = static_cast<bf16>(acc.x); o.b[1] = static_cast<bf16>(acc.y);
+      o.b[2] = static_cast<bf16>(acc.z); o.b[3] = static_cast<bf16>(acc.w);
+      *reinterpret_cast<uint2*>(&xs[m][j * D + d]) = o.u;
+    }
+  }
+  __syncthreads();
+  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < STEPS; ++u) {
+    if (u * 64 < KB) {
+      const bf16* xp = &xs[r][u * 64 + g * 16];
+      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp);
+      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + 8);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][0].v, x0, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][1].v, x1, acc, 0, 0, 0);
+    }
+  }
+  // acc[e] = Y[m = r][n = nb + 4 g + e] of this block's heads
+  if (r < rows && row_in)
+    *reinterpret_cast<float4*>(P + ((size_t)blockIdx.x * rows + r) * N + nb + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+}
+
+// Heads per block so that the output projection's partial sums number at most 16.
+extern "C" int ms_attention_merge_project_splits(int Hq) {
+  const int hb = (Hq + 15) / 16;
+  return hb > MERGE_MAX_HB || Hq % hb ? -1 : Hq / hb;
+}
+
+// P [ms_attention_merge_project_splits(Hq), rows, N] (float partial sums) from the split attention's
+// partial results of `rows` <= 16 single-token rows (part_o, part_ml as the decode kernels leave them)
+// and the output projection's weight W [N, Hq * D]. MS_UNSUPPORTED where the two separate kernels must run.
+extern "C" int ms_attention_merge_project(const float* part_o, const float* part_ml, const void* W, float* P, int rows,
+                                          int Hq, int D, int splits, int N, hipStream_t st) {
+  if (rows <= 0 || N <= 0) return MS_OK;
+  if (part_o == nullptr || part_ml == nullptr || W == nullptr || P == nullptr || Hq <= 0 || splits < 1) return MS_BAD_ARG;
+  const int out_splits = ms_attention_merge_project_splits(Hq);
+  if (rows > 16 || splits > MERGE_MAX_SPLITS || (D != 64 && D != 128) || N % 64 || out_splits < 1) return MS_UNSUPPORTED;
+  const int hb = Hq / out_splits;
+  if ((hb * D) % 64) return MS_UNSUPPORTED;
+  dim3 grid(out_splits, N / 64);
+  if (D == 128) attn_merge_project_kernel<128, 4><<<grid, 256, 0, st>>>(part_o, part_ml, (const bf16*)W, P, rows, Hq, splits, hb, N);
+  else attn_merge_project_kernel<64, 4><<<grid, 256, 0, st>>>(part_o, part_ml, (const bf16*)W, P, rows, Hq, splits, hb, N);
+  return launch_status();
 }

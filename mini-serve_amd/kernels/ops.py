@@ -44,7 +44,9 @@ _SIGNATURES = {
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_void,
                                        _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
-                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
+    "ms_attention_merge_project": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_attention_merge_project_splits": [_c_int],
     "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
                                   _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_parts_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void,
@@ -487,12 +489,22 @@ def decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_ca
             and (rope is None or rope.shape[1] == head_dim))
 
 
+MERGE_PROJECT_MAX_ROWS = 16  # rows up to which the splits' reduction and the output projection are one kernel
+MERGE_PROJECT_MAX_SPLITS = 64
+
+
 def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v_cache, block_table, batch,
-                           num_heads, num_kv_heads, head_dim, scale, window) -> torch.Tensor:
+                           num_heads, num_kv_heads, head_dim, scale, window, project: torch.Tensor | None = None):
     """``qk_norm_rope_store`` and ``paged_attention`` of a step of single tokens in one kernel, from the
     partial sums ``qkv`` (a ``SplitSum`` of ``[T, (Hq + 2 Hkv) D]``): the queries never go to memory,
     and with ``store`` the new token's key and value are written to the cache by the block that uses
-    them first. Returns bfloat16 ``[T, Hq * D]``. ``decode_attention_fusable`` says when this applies."""
+    them first. Returns bfloat16 ``[T, Hq * D]``. ``decode_attention_fusable`` says when this applies.
+
+    ``project``: the output projection's weight ``[N, Hq * D]`` (bfloat16). Where the keys were split
+    (they are whenever the step has few rows) and the step has up to ``MERGE_PROJECT_MAX_ROWS`` rows,
+    the reduction of the splits and that projection run as one kernel and a ``SplitSum`` of
+    ``[T, N]`` is returned instead of the attention's output: no reduction kernel, and the attention's
+    output never goes to memory."""
     if not decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim):
         raise ValueError("this step cannot run the fused decode attention")
     _dev(qkv.parts, "qkv", F32, 3)
@@ -516,18 +528,33 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
     _dev(batch.positions, "positions", I32, 1)
     if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
         raise ValueError("batch metadata does not match the number of tokens or rows")
-    out = torch.empty((t, num_heads * head_dim), dtype=BF16, device=qkv.parts.device)
+    dev = qkv.parts.device
+    lib = library()
     splits = decode_splits(t, num_kv_heads, batch.max_kv_len)
     part_o = part_ml = None
     if splits > 1:
-        part_o = torch.empty((t * num_heads * splits * head_dim,), dtype=F32, device=out.device)
-        part_ml = torch.empty((t * num_heads * splits * 2,), dtype=F32, device=out.device)
-    _check(library().ms_attention_decode_fused_bf16(
+        part_o = torch.empty((t * num_heads * splits * head_dim,), dtype=F32, device=dev)
+        part_ml = torch.empty((t * num_heads * splits * 2,), dtype=F32, device=dev)
+    merged = None  # partial sums of the projection, where one kernel reduces the splits and projects
+    if (project is not None and MERGE_PROJECT_MAX_ROWS > 0 and 1 < splits <= MERGE_PROJECT_MAX_SPLITS
+            and t <= MERGE_PROJECT_MAX_ROWS):
+        _dev(project, "project", BF16, 2)
+        n = project.shape[0]
+        out_splits = lib.ms_attention_merge_project_splits(num_heads)
+        if project.shape[1] == num_heads * head_dim and n % 64 == 0 and out_splits >= 1:
+            merged = torch.empty((out_splits, t, n), dtype=F32, device=dev)
+    out = None if merged is not None else torch.empty((t, num_heads * head_dim), dtype=BF16, device=dev)
+    _check(lib.ms_attention_decode_fused_bf16(
         qkv.parts.data_ptr(), qkv.splits, qkv.stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(rope), int(bool(store)),
         k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], None,
-        batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml), t, splits,
-        num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "attention_decode_fused")
-    return out
+        batch.token_row.data_ptr(), batch.positions.data_ptr(), _ptr(out), _ptr(part_o), _ptr(part_ml), t, splits,
+        num_heads, num_kv_heads, head_dim, page, float(scale), int(window), int(merged is None), _stream()),
+        "attention_decode_fused")
+    if merged is None:
+        return out
+    _check(lib.ms_attention_merge_project(part_o.data_ptr(), part_ml.data_ptr(), project.data_ptr(), merged.data_ptr(), t,
+                                          num_heads, head_dim, splits, merged.shape[2], _stream()), "attention_merge_project")
+    return SplitSum(merged)
 
 
 def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window):

@@ -92,11 +92,14 @@ class GQAttention(Mixer):
         if ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
                                         self.heads, self.kv_heads, self.head_dim):
             # a step of single tokens: norm, rotation, cache store and attention are one kernel
+            # ... and, with few rows, the reduction of the key splits and the output projection another
             out = ops.decode_attention_fused(
                 qkv, self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps), table,
                 cache.writes, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
-                self.scale, self.window,
+                self.scale, self.window, project=self.o if self.o.dtype == torch.bfloat16 else None,
             )
+            if isinstance(out, ops.SplitSum):
+                return out  # the projection's partial sums: pending, for the next reader of the stream
             return ops.linear(out, self.o, accumulate_into=residual, defer=True)
         q = ops.qk_norm_rope_store(
             qkv, cache.slots if cache.writes else None,

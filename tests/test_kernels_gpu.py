@@ -84,6 +84,34 @@ def test_rmsnorm_adds_partial_sums(ops, width, splits, out_dtype):
     assert torch.equal(x2, x)
 
 
+@pytest.mark.parametrize("width", [256, 1024, 2304, 5120, 8192, 1000])
+@pytest.mark.parametrize("w_dtype", [F32, BF16])
+def test_rmsnorm_of_many_rows(ops, width, w_dtype):
+    """More than 64 rows with bfloat16 output (a prompt's portion) run a wave per row; with and without
+    partial sums to add, all rows or a list of them."""
+    m, eps = 301, 1e-5
+    x = rand((m, width), F32, 5, 2.0)
+    w = rand((width,), w_dtype, 6) + 1
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps) * w.double()
+    close(ops.rmsnorm(x, w, eps, BF16), want, 5e-3, "many rows")
+    rows = torch.arange(m - 1, -1, -3, dtype=torch.int32, device=DEV)
+    assert rows.shape[0] > 64
+    close(ops.rmsnorm(x, w, eps, BF16, rows), want[rows.long()], 5e-3, "a long row list")
+    # a row's bits do not depend on how many rows came with it (beyond 64)
+    assert torch.equal(ops.rmsnorm(x, w, eps, BF16)[:70], ops.rmsnorm(x[:70].contiguous(), w, eps, BF16))
+    for splits in (2, 5):
+        parts = rand((splits, m, width), F32, 7)
+        full = xd + parts.double().sum(0)
+        wantp = full / torch.sqrt((full * full).mean(-1, keepdim=True) + eps) * w.double()
+        x1 = x.clone()
+        close(ops.rmsnorm(x1, w, eps, BF16, add=ops.SplitSum(parts)), wantp, 5e-3, f"{splits} partial sums")
+        close(x1, full, 1e-6, "stream brought up to date")
+        x2 = x.clone()
+        close(ops.rmsnorm(x2, w, eps, BF16, rows, add=ops.SplitSum(parts)), wantp[rows.long()], 5e-3, "row list with partial sums")
+        assert torch.equal(x2, x)
+
+
 def test_rmsnorm_eps_enters(ops):
     x = rand((2, 64), F32, 4, 1e-3)
     w = torch.ones(64, device=DEV)
@@ -570,6 +598,22 @@ def test_decode_attention_fused(ops, hq, hkv, d, starts, window, norm, rot):
     got = ops.decode_attention_fused(ops.SplitSum(parts), qw, kw, eps, rope, False, k3, v3, table, batch, hq, hkv, d, scale, window)
     close(got, want, 8e-3, "fused decode attention without the store")
     assert torch.equal(k3, k1) and torch.equal(v3, v1)
+
+    # with the output projection's weight: up to 16 rows whose keys are split come back as the projection's
+    # partial sums (the reduction of the splits and the projection are one kernel)
+    n = 192
+    wo = rand((n, hq * d), BF16, 86, 0.05)
+    k4, v4 = kc.clone(), vc.clone()
+    got = ops.decode_attention_fused(ops.SplitSum(parts), qw, kw, eps, rope, True, k4, v4, table, batch, hq, hkv, d, scale, window,
+                                     project=wo)
+    splits = ops.decode_splits(b, hkv, batch.max_kv_len)
+    if b <= 16 and 1 < splits <= 64:
+        assert isinstance(got, ops.SplitSum) and got.shape == (b, n) and got.splits <= 16
+        close(got.parts.double().sum(0), want.double() @ wo.double().T, 1e-2, "reduction of the splits and projection in one")
+        assert torch.equal(k4, k2.nan_to_num(0)) or torch.equal(flat(k4, False)[sl], flat(k2, False)[sl])
+    else:
+        assert isinstance(got, torch.Tensor)
+        close(got, want, 8e-3, "no projection where the keys are not split or the rows are many")
 
 
 def test_decode_splits_rule(ops):
