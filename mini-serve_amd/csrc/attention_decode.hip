@@ -499,38 +499,36 @@ extern "C" int ms_attention_decode_fused_bf16(const float* parts, int qkv_splits
 // of few rows. At most 64 splits (a lane each).
 #define MERGE_MAX_SPLITS 64
 #define MERGE_MAX_HB 4
-template <int D, int NW>
-__global__ __launch_bounds__(NW * WAVE) void attn_merge_project_kernel(const float* __restrict__ part_o,
-                                                                       const float* __restrict__ part_ml,
-                                                                       const bf16* __restrict__ W, float* __restrict__ P,
-                                                                       int rows, int Hq, int splits, int HB, int N) {
-  __shared__ float fw[MERGE_MAX_HB][16][MERGE_MAX_SPLITS];            // weight of split s in row m of head j
-  __shared__ __attribute__((aligned(16))) bf16 xs[16][MERGE_MAX_HB * D + 8];  // merged rows; rows beyond `rows` are zero
+// HB heads per block; every wave takes NPW blocks of 16 rows of W (so that a wide W does not mean many
+// blocks that each merge the same splits again).
+template <int D, int HB, int NPW>
+__global__ __launch_bounds__(256) void attn_merge_project_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 const bf16* __restrict__ W, float* __restrict__ P, int rows,
+                                                                 int Hq, int splits, int N) {
+  constexpr int NW = 4, KB = HB * D, STEPS = KB / 64;
+  __shared__ float fw[HB][16][MERGE_MAX_SPLITS];                 // weight of split s in row m of head j
+  __shared__ __attribute__((aligned(16))) bf16 xs[16][KB + 8];   // merged rows; rows beyond `rows` are zero
   __shared__ float4 psum[NW * WAVE];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int h0 = blockIdx.x * HB;          // first head of this block
-  const int K = Hq * D, KB = HB * D;       // columns of W; of this block
-  const int nb = (blockIdx.y * NW + wave) * 16;
+  const int h0 = blockIdx.x * HB;  // first head of this block
+  const int K = Hq * D;            // columns of W
+  const int nb0 = (blockIdx.y * NW + wave) * NPW * 16;
   // weights first: they come from memory, everything below from the cache
-  constexpr int STEPS = MERGE_MAX_HB * D / 64;
   union Chunk { uint4 u; bf16x8 v; };
-  Chunk a[STEPS][2];
-  const bool row_in = nb + 16 <= N;
-  {
-    const bf16* wp = W + (size_t)min(nb + r, N - 1) * K + (size_t)h0 * D + g * 16;
+  Chunk a[NPW][STEPS][2];
+#pragma unroll
+  for (int q = 0; q < NPW; ++q) {
+    const bf16* wp = W + (size_t)min(nb0 + q * 16 + r, N - 1) * K + (size_t)h0 * D + g * 16;
 #pragma unroll
     for (int u = 0; u < STEPS; ++u) {
-      if (u * 64 < KB) {
-        a[u][0].u = *reinterpret_cast<const uint4*>(wp + u * 64);
-        a[u][1].u = *reinterpret_cast<const uint4*>(wp + u * 64 + 8);
-      } else {
-        a[u][0].u = a[u][1].u = make_uint4(0, 0, 0, 0);
-      }
+      a[q][u][0].u = *reinterpret_cast<const uint4*>(wp + u * 64);
+      a[q][u][1].u = *reinterpret_cast<const uint4*>(wp + u * 64 + 8);
     }
   }
-  for (int e = tid; e < 16 * MERGE_MAX_HB * (D / 4); e += NW * WAVE)  // rows beyond `rows` and heads beyond HB read as zero
-    *reinterpret_cast<uint2*>(&xs[e / (MERGE_MAX_HB * (D / 4))][(e % (MERGE_MAX_HB * (D / 4))) * 4]) = make_uint2(0, 0);
+  for (int e = tid; e < 16 * (KB / 4); e += NW * WAVE)  // rows beyond `rows` read as zero
+    *reinterpret_cast<uint2*>(&xs[e / (KB / 4)][(e % (KB / 4)) * 4]) = make_uint2(0, 0);
   // the weights of the splits: wave w takes the (row, head) pairs w, w + NW, ...
   for (int p = wave; p < rows * HB; p += NW) {
     const int m = p / HB, j = p % HB;
@@ -590,20 +588,26 @@ __global__ __launch_bounds__(NW * WAVE) void attn_merge_project_kernel(const flo
     }
   }
   __syncthreads();
-  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 x[STEPS][2];
 #pragma unroll
   for (int u = 0; u < STEPS; ++u) {
-    if (u * 64 < KB) {
-      const bf16* xp = &xs[r][u * 64 + g * 16];
-      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp);
-      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + 8);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][0].v, x0, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][1].v, x1, acc, 0, 0, 0);
-    }
+    const bf16* xp = &xs[r][u * 64 + g * 16];
+    x[u][0] = *reinterpret_cast<const bf16x8*>(xp);
+    x[u][1] = *reinterpret_cast<const bf16x8*>(xp + 8);
   }
-  // acc[e] = Y[m = r][n = nb + 4 g + e] of this block's heads
-  if (r < rows && row_in)
-    *reinterpret_cast<float4*>(P + ((size_t)blockIdx.x * rows + r) * N + nb + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+#pragma unroll
+  for (int q = 0; q < NPW; ++q) {
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[q][u][0].v, x[u][0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[q][u][1].v, x[u][1], acc, 0, 0, 0);
+    }
+    // acc[e] = Y[m = r][n = nb + 4 g + e] of this block's heads
+    const int nb = nb0 + q * 16;
+    if (r < rows && nb + 16 <= N)
+      *reinterpret_cast<float4*>(P + ((size_t)blockIdx.x * rows + r) * N + nb + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  }
 }
 
 // Heads per block so that the output projection's partial sums number at most 16.
@@ -622,9 +626,21 @@ extern "C" int ms_attention_merge_project(const float* part_o, const float* part
   const int out_splits = ms_attention_merge_project_splits(Hq);
   if (rows > 16 || splits > MERGE_MAX_SPLITS || (D != 64 && D != 128) || N % 64 || out_splits < 1) return MS_UNSUPPORTED;
   const int hb = Hq / out_splits;
-  if ((hb * D) % 64) return MS_UNSUPPORTED;
-  dim3 grid(out_splits, N / 64);
-  if (D == 128) attn_merge_project_kernel<128, 4><<<grid, 256, 0, st>>>(part_o, part_ml, (const bf16*)W, P, rows, Hq, splits, hb, N);
-  else attn_merge_project_kernel<64, 4><<<grid, 256, 0, st>>>(part_o, part_ml, (const bf16*)W, P, rows, Hq, splits, hb, N);
+  if ((hb * D) % 64 || (hb != 1 && hb != 2 && hb != 4)) return MS_UNSUPPORTED;
+  // Rows of W per block: 64, or 256 where that still leaves a block for every CU.
+  const int npw = (N % 256 == 0 && (long)out_splits * (N / 256) >= 256) ? 4 : 1;
+  dim3 grid(out_splits, N / (64 * npw));
+  const bf16* w = (const bf16*)W;
+#define LAUNCH(DD, HB, NPW) attn_merge_project_kernel<DD, HB, NPW><<<grid, 256, 0, st>>>(part_o, part_ml, w, P, rows, Hq, splits, N)
+#define LAUNCH_HB(DD, NPW)                                                                                              \
+  if (hb == 1) LAUNCH(DD, 1, NPW);                                                                                      \
+  else if (hb == 2) LAUNCH(DD, 2, NPW);                                                                                 \
+  else LAUNCH(DD, 4, NPW)
+  if (D == 128 && npw == 4) { LAUNCH_HB(128, 4); }
+  else if (D == 128) { LAUNCH_HB(128, 1); }
+  else if (npw == 4) { LAUNCH_HB(64, 4); }
+  else { LAUNCH_HB(64, 1); }
+#undef LAUNCH_HB
+#undef LAUNCH
   return launch_status();
 }

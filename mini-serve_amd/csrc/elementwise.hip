@@ -175,62 +175,6 @@ __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x,
   }
 }
 
-// Many rows (a prompt's portion) of a width that is a multiple of 256 and at most 8192, bfloat16 output: a
-// wave per row, four rows per block. A lane owns groups of 4 consecutive elements 256 apart (a wave's
-// load covers 1 KB of the row at once), the row's sum of squares is a wave reduction: no LDS, no
-// barrier, and every load of a row is issued before the first is used. Partial sums as above.
-template <typename TW, int GROUPS>
-__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(float* __restrict__ x, const TW* __restrict__ w,
-                                                            bf16* __restrict__ y, const int* __restrict__ rows, int n_rows,
-                                                            int width, float eps, const float* __restrict__ parts, int splits,
-                                                            size_t split_stride) {
-  const int lane = threadIdx.x % WAVE;
-  const int r = blockIdx.x * 4 + threadIdx.x / WAVE;
-  if (r >= n_rows) return;
-  const size_t row = rows ? rows[r] : r;
-  float* src = x + row * width;
-  const bool in_place = parts != nullptr && rows == nullptr;
-  const int groups = width / 256;  // <= GROUPS
-  float4 kept[GROUPS];
-#pragma unroll
-  for (int j = 0; j < GROUPS; ++j)
-    kept[j] = j < groups ? *reinterpret_cast<const float4*>(src + j * 256 + lane * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-  float ss = 0.f;
-#pragma unroll
-  for (int j = 0; j < GROUPS; ++j) {
-    float4 v = kept[j];
-    if (parts != nullptr && j < groups) {
-      const float* p = parts + row * width + j * 256 + lane * 4;
-      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (splits <= 2) {
-        add_splits<2>(acc, p, 0, splits, split_stride);
-      } else if (splits <= 4) {
-        add_splits<4>(acc, p, 0, splits, split_stride);
-      } else {
-        for (int s0 = 0; s0 < splits; s0 += 8) add_splits<8>(acc, p, s0, splits, split_stride);
-      }
-      v.x += acc.x; v.y += acc.y; v.z += acc.z; v.w += acc.w;
-      if (in_place) *reinterpret_cast<float4*>(src + j * 256 + lane * 4) = v;
-      kept[j] = v;
-    }
-    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-  }
-  ss = wave_sum(ss);
-  const float rstd = rsqrtf(ss / (float)width + eps);
-  bf16* dst = y + (size_t)r * width;
-#pragma unroll
-  for (int j = 0; j < GROUPS; ++j) {
-    if (j >= groups) break;
-    const int i = j * 256 + lane * 4;
-    union { uint2 u; bf16 e[4]; } o;
-    o.e[0] = from_f32<bf16>(kept[j].x * rstd * to_f32(w[i]));
-    o.e[1] = from_f32<bf16>(kept[j].y * rstd * to_f32(w[i + 1]));
-    o.e[2] = from_f32<bf16>(kept[j].z * rstd * to_f32(w[i + 2]));
-    o.e[3] = from_f32<bf16>(kept[j].w * rstd * to_f32(w[i + 3]));
-    *reinterpret_cast<uint2*>(dst + i) = o.u;
-  }
-}
-
 extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y_is_bf16, const int* rows, int n_rows,
                           int width, float eps, const float* parts, int splits, long long split_stride, hipStream_t st) {
   if (n_rows <= 0) return MS_OK;
@@ -238,21 +182,6 @@ extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y
   // float32 output keeps one block shape for every batch, so that its sums are formed in one order
   // whatever the batch; bfloat16 output takes the wide block for few rows.
   const bool wide = y_is_bf16 && n_rows <= 256;
-  // Which kernel runs depends on the class of the row count (up to 64, more), never on the rows themselves.
-  if (y_is_bf16 && n_rows > 64 && width % 256 == 0 && width <= 8192 && (parts == nullptr || split_stride % 4 == 0)) {
-#define LAUNCH_ROWS(TW, G)                                                                                              \
-  rmsnorm_rows_kernel<TW, G><<<(n_rows + 3) / 4, 256, 0, st>>>(x, (const TW*)w, (bf16*)y, rows, n_rows, width, eps, parts, \
-                                                                splits, (size_t)split_stride)
-#define LAUNCH_ROWS_W(TW)                                                                                               \
-  if (width <= 1024) { LAUNCH_ROWS(TW, 4); }                                                                            \
-  else if (width <= 2048) { LAUNCH_ROWS(TW, 8); }                                                                       \
-  else if (width <= 4096) { LAUNCH_ROWS(TW, 16); }                                                                      \
-  else { LAUNCH_ROWS(TW, 32); }
-    if (w_is_bf16) { LAUNCH_ROWS_W(bf16) } else { LAUNCH_ROWS_W(float) }
-#undef LAUNCH_ROWS_W
-#undef LAUNCH_ROWS
-    return launch_status();
-  }
   if (y_is_bf16 && width % 4 == 0 && width <= 8192 && (parts == nullptr || split_stride % 4 == 0)) {
 #define LAUNCH_VEC(TW)                                                                                                  \
   if (width <= 2048)                                                                                                    \

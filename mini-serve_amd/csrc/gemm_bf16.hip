@@ -241,17 +241,20 @@ __device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int co
   return id;
 }
 
-template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
-__global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+// WR x WC waves per block, each with a wave tile of BM / WR x BN / WC.
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU, int WR = 2, int WC = 2>
+__global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
                                                                int ldx, int ldc, int k_per, size_t c_split_stride, int xcd_rows,
                                                                int band_cols) {
-  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int NW = WR * WC;
+  constexpr int WM = BM / WR, WN = BN / WC;
   constexpr int FM = WM / 16, FN = WN / 16;
   constexpr int ROW_BYTES = KS * 2;           // a tile row: KS k of bf16
   constexpr int CPR = KS / 8;                 // 16-byte chunks per row
   constexpr int RPI = 1024 / ROW_BYTES;       // rows a load instruction of a wave fills
-  constexpr int XI = BM / (4 * RPI), WI = BN / (4 * RPI);  // load instructions per wave and slab
+  constexpr int XI = BM / (NW * RPI), WI = BN / (NW * RPI);  // load instructions per wave and slab
+  static_assert(BM % (NW * RPI) == 0 && BN % (NW * RPI) == 0, "every wave loads whole instructions of both operands");
   constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // STAGES * STAGE_BYTES
 
@@ -259,7 +262,7 @@ __global__ __launch_bounds__(256, BLOCKS_PER_CU) void gemm_bf16_dma_kernel(const
   const int r = lane % 16, g = lane / 16;
   const TileId id = tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, xcd_rows, band_cols);
   const int m0 = id.m * BM, n0 = id.n * BN;
-  const int wm = (wave / 2) * WM, wn = (wave % 2) * WN;
+  const int wm = (wave / WC) * WM, wn = (wave % WC) * WN;
   const int k_lo = id.split * k_per;
   const int K = min(Kfull, k_lo + k_per);
   const int slabs = (K - k_lo) / KS;
@@ -544,13 +547,13 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
 // bound by memory; with them at 850-950.
 constexpr long DMA_BAND_BYTES = 96L << 20;
 
-template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU>
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU, int WR = 2, int WC = 2>
 static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
                       size_t stride, int splits, hipStream_t st) {
   constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
   static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
   if (!ready) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU>,
+    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
       return MS_LAUNCH_FAILED;
     ready = true;
@@ -589,8 +592,21 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
     const long bands = (sub_cols + band_cols - 1) / band_cols;
     band_cols = (sub_cols + bands - 1) / bands;
   }
-  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU><<<(unsigned)blocks, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, xcd_rows, (int)band_cols);
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC><<<(unsigned)blocks, WR * WC * WAVE, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, xcd_rows, (int)band_cols);
   return launch_status();
+}
+
+// 256 x 256 tiles of eight waves (4 x 2, wave tiles of 64 x 128, one block per CU with all 256 registers
+// and 128 KB of LDS): a wave reads 12 fragments for 32 products where the 64 x 64 wave tile of the
+// 128-row blocks reads 8 for 16, so the fragment reads no longer take as long as the products. They pay
+// where they fill the chip: at least one round of 256 blocks and no round less than three quarters full
+// (measured against the 128-row tiles: 8192^3 1210 against 1120 TFLOP/s, 4096^3 1150 against 1030,
+// 2048 x 51200 x 5120 1100 against 980, 512 x 51200 x 5120 960 against 890; with 128 tiles at
+// 2048 x 4096 x 4096 600 against 900).
+static bool huge_tiles_pay(int M, int N, int splits) {
+  const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256) * splits;
+  const long rounds = (tiles + 255) / 256;
+  return tiles >= 256 && tiles * 4 >= rounds * 256 * 3;
 }
 
 // Width of the 128-row tiles of a product: 64, 128 or 192 columns. All blocks of up to 512 (two per CU)
@@ -808,6 +824,7 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
     return MS_UNSUPPORTED;
   }
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (huge_tiles_pay(M, N, 1)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
   if (big >= 256) {
     const int cols = wide_tile_cols(M, N, 1);
     if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
@@ -878,6 +895,7 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
   // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
   if (K % BK == 0 && ldx % 8 == 0) {
+    if (huge_tiles_pay(M, N, splits)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     if (big >= 256) {
       const int cols = wide_tile_cols(M, N, splits);
       if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
