@@ -8,7 +8,6 @@ Tensors are torch tensors used as plain device buffers; no torch operator comput
 from __future__ import annotations
 
 import ctypes
-import os
 
 import torch
 

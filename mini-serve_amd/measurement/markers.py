@@ -2,11 +2,12 @@
 NVTX ranges so that a profile holds those steps and nothing of the set-up
 (bench/offline.py:235-241,435,443-445); here the same with the ROCTx library that ships with ROCm:
 
-    rocprofv3 --kernel-trace --stats --selected-regions -- python3 bench.py ...
+    rocprofv3 --kernel-trace --marker-trace --stats --selected-regions -- python3 bench.py ...
 
 keeps only what runs inside ``measured_region`` (it calls ``roctxProfilerResume`` on entry and
-``roctxProfilerPause`` on exit); ``--marker-trace`` shows the named ranges of ``mark``. Without the
-library, or outside a profiler, every call is a no-op."""
+``roctxProfilerPause`` on exit; without ``--marker-trace`` the profiler does not see these calls and
+records nothing); the marker trace also shows the named ranges of ``mark``. Without the library, or
+outside a profiler, every call is a no-op."""
 
 from __future__ import annotations
 
