@@ -602,11 +602,13 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
 // where they fill the chip: at least one round of 256 blocks and no round less than three quarters full
 // (measured against the 128-row tiles: 8192^3 1210 against 1120 TFLOP/s, 4096^3 1150 against 1030,
 // 2048 x 51200 x 5120 1100 against 980, 512 x 51200 x 5120 960 against 890; with 128 tiles at
-// 2048 x 4096 x 4096 600 against 900).
-static bool huge_tiles_pay(int M, int N, int splits) {
+// 2048 x 4096 x 4096 600 against 900), and, with a long K, from 160 tiles on (2048 x 5120 x 25600: 860
+// against 780; x 8192: 860 against 800).
+static bool huge_tiles_pay(int M, int N, int K, int splits) {
   const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256) * splits;
   const long rounds = (tiles + 255) / 256;
-  return tiles >= 256 && tiles * 4 >= rounds * 256 * 3;
+  if (tiles >= 256 && tiles * 4 >= rounds * 256 * 3) return true;
+  return tiles >= 160 && tiles <= 256 && K / splits >= 8192;
 }
 
 // Width of the 128-row tiles of a product: 64, 128 or 192 columns. All blocks of up to 512 (two per CU)
@@ -824,7 +826,7 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
     return MS_UNSUPPORTED;
   }
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (huge_tiles_pay(M, N, 1)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  if (huge_tiles_pay(M, N, K, 1)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
   if (big >= 256) {
     const int cols = wide_tile_cols(M, N, 1);
     if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
@@ -895,7 +897,7 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
   // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
   if (K % BK == 0 && ldx % 8 == 0) {
-    if (huge_tiles_pay(M, N, splits)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    if (huge_tiles_pay(M, N, K, splits)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     if (big >= 256) {
       const int cols = wide_tile_cols(M, N, splits);
       if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
