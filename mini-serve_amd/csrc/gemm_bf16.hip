@@ -343,10 +343,10 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
   if (mode == 3) {
     // Gated epilogue: W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and
     // 2 p + 1 of a lane are gate and up of the same four outputs: out[m, n / 2 ...] = silu(gate) * up,
-    // bf16 [M, N / 2] with row stride ldc.
-    static_assert(FN % 2 == 0, "gate and up fragments come in pairs");
+    // bf16 [M, N / 2] with row stride ldc. Wave tiles with an odd number of fragments are never
+    // launched in this mode.
 #pragma unroll
-    for (int i = 0; i < FN; i += 2)
+    for (int i = 0; i + 1 < FN; i += 2)
 #pragma unroll
       for (int j = 0; j < FM; ++j) {
         const int m = m0 + wm + j * 16 + r, col = (n0 + wn + i * 16) / 2 + g * 4;
@@ -596,41 +596,62 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
   return launch_status();
 }
 
-// 256 x 256 tiles of eight waves (4 x 2, wave tiles of 64 x 128, one block per CU with all 256 registers
-// and 128 KB of LDS): a wave reads 12 fragments for 32 products where the 64 x 64 wave tile of the
-// 128-row blocks reads 8 for 16, so the fragment reads no longer take as long as the products. They pay
-// where they fill the chip: at least one round of 256 blocks and no round less than three quarters full
-// (measured against the 128-row tiles: 8192^3 1210 against 1120 TFLOP/s, 4096^3 1150 against 1030,
-// 2048 x 51200 x 5120 1100 against 980, 512 x 51200 x 5120 960 against 890; with 128 tiles at
-// 2048 x 4096 x 4096 600 against 900), and, with a long K, from 160 tiles on (2048 x 5120 x 25600: 860
-// against 780; x 8192: 860 against 800).
-static bool huge_tiles_pay(int M, int N, int K, int splits) {
-  const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256) * splits;
-  const long rounds = (tiles + 255) / 256;
-  if (tiles >= 256 && tiles * 4 >= rounds * 256 * 3) return true;
-  return tiles >= 160 && tiles <= 256 && K / splits >= 8192;
-}
+// Tile shape of a product with at least 256 tiles of 128 x 128: 128-row tiles of four waves, 64 to 192
+// columns wide, two blocks per CU (512 run at once), or 256 x 256 tiles of eight waves (4 x 2, wave
+// tiles of 64 x 128, one block per CU with all 256 registers and 128 KB of LDS: a wave reads 12
+// fragments for 32 products where the 64 x 64 wave tile reads 8 for 16). The choice is the least
+// predicted time: a fixed part (launch, first slab, stores) plus, per slab of 64 k, the time of a round
+// of blocks. A block that has a CU to itself is faster than one that shares it, so a last round of up
+// to 256 blocks counts less than a full one. The figures (microseconds) are a fit to 270 products
+// (384 to 8,192 rows, 1,024 to 24,576 columns, K of 1,024, 4,096 and 12,288) timed with every shape;
+// picking by them is within 1 % of the best shape on average and 17 % at worst, where rules by tile
+// counts alone lost up to 28 % (2,048 x 5,120 x 12,288: 160 columns make exactly 512 tiles).
+struct TileShape {
+  int cols;      // 256 stands for the 256 x 256 tile
+  float fixed;   // per launch
+  float alone;   // per slab, a last round with one block per CU
+  float shared;  // per slab, a round with two blocks per CU
+};
+static const TileShape TILE_SHAPES[5] = {
+    {128, 7.7f, 0.611f, 0.976f}, {64, 6.1f, 0.456f, 0.627f}, {160, 8.8f, 0.707f, 1.168f},
+    {192, 9.1f, 0.803f, 1.364f}, {256, 12.6f, 1.476f, 1.476f}};
 
-// Width of the 128-row tiles of a product: 64, 128 or 192 columns. All blocks of up to 512 (two per CU)
-// run at once, so what counts is how many such rounds the tiles make and how long a tile of each width
-// takes (measured at 2,048 rows, relative to 128 columns): a 192-wide tile does 1.5 times the work in
-// 1.4 times the time, a 64-wide one half the work in 0.62; a few rounds count whole, many as they are.
-static int wide_tile_cols(int M, int N, int splits) {
-  const int widths[3] = {128, 192, 64};
-  const double tile_time[3] = {1.0, 1.4, 0.62};
-  const long row_tiles = (M + 127) / 128;
+// `pairs`: the gated epilogue needs an even number of 16-column fragments per wave, which 160 columns
+// over two waves are not.
+static int pick_tile_cols(int M, int N, int K, int splits, bool pairs) {
+  const float slabs = (float)((K + BK - 1) / BK) / splits;
   int best = 128;
-  double least = 0;
-  for (int i = 0; i < 3; ++i) {
-    const long tiles = row_tiles * ((N + widths[i] - 1) / widths[i]) * splits;
-    const double rounds = tiles <= 1024 ? (double)((tiles + 511) / 512) : tiles / 512.0;
-    const double t = rounds * tile_time[i];
-    if (i == 0 || t < least * 0.97) {  // another width has to be clearly better
-      least = t;
-      best = widths[i];
+  float least = 0.f;
+  for (int i = 0; i < 5; ++i) {
+    const TileShape& t = TILE_SHAPES[i];
+    if (pairs && t.cols == 160) continue;
+    float rounds;
+    if (t.cols == 256) {
+      const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256) * splits;
+      rounds = (float)((tiles + 255) / 256) * t.shared;
+    } else {
+      const long tiles = (long)((M + 127) / 128) * ((N + t.cols - 1) / t.cols) * splits;
+      const long rest = tiles % 512;
+      rounds = (float)(tiles / 512) * t.shared + (rest == 0 ? 0.f : rest <= 256 ? t.alone : t.shared);
+    }
+    const float time = t.fixed + slabs * rounds;
+    if (i == 0 || time < least) {
+      least = time;
+      best = t.cols;
     }
   }
   return best;
+}
+
+static int launch_picked(int cols, const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc,
+                         int k_per, size_t stride, int splits, hipStream_t st) {
+  switch (cols) {
+    case 256: return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    case 192: return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    case 160: return launch_dma<128, 160, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    case 64: return launch_dma<128, 64, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    default: return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+  }
 }
 
 // Splits of K for the small-M kernel: one slab (four 64-k steps) per wave, so that a wave issues all
@@ -826,13 +847,7 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
     return MS_UNSUPPORTED;
   }
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (huge_tiles_pay(M, N, K, 1)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
-  if (big >= 256) {
-    const int cols = wide_tile_cols(M, N, 1);
-    if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
-    if (cols == 64) return launch_dma<128, 64, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
-    return launch_dma<128, 128, BK, 2, 2>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
-  }
+  if (big >= 256) return launch_picked(pick_tile_cols(M, N, K, 1, true), x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
   // 64 x 64 tiles from 128 of them on: half the CUs without a split of K still beat the split product
   // followed by the activation kernel (10.2 against 11.8 to 13.1 us at 65 to 128 rows of the 0.6B shape).
   if ((long)((M + 63) / 64) * ((N + 63) / 64) >= 128) return launch_dma<64, 64, BK, 2, 4>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
@@ -897,13 +912,8 @@ extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int
   // shapes tried at M = 2048 (tiles 128 or 256 wide, slabs of 32 or 64 k, 2 to 4 stages, 1 to 4 blocks
   // per CU) 128 x 128 tiles with two stages of 64 k and two blocks per CU were fastest throughout.
   if (K % BK == 0 && ldx % 8 == 0) {
-    if (huge_tiles_pay(M, N, K, splits)) return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
-    if (big >= 256) {
-      const int cols = wide_tile_cols(M, N, splits);
-      if (cols == 192) return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
-      if (cols == 64) return launch_dma<128, 64, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
-      return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
-    }
+    if (big >= 256)
+      return launch_picked(pick_tile_cols(M, N, K, splits, false), x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     return launch_dma<64, 64, BK, 2, 4>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
   }
   if (big >= 256) {

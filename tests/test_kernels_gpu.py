@@ -169,16 +169,20 @@ def test_gemm_bf16(ops, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024),
                                    (4000, 1500, 192), (1990, 1000, 128), (2048, 6100, 128), (2048, 1000, 256),
-                                   (5000, 5000, 128), (4096, 4096, 64), (600, 33000, 192)])
+                                   (5000, 5000, 128), (4096, 4096, 64), (600, 33000, 192),
+                                   (1990, 5100, 512), (4100, 1000, 512), (4000, 4200, 1024), (600, 33000, 512),
+                                   (4090, 4090, 1024), (3000, 5000, 1024)])
 def test_gemm_bf16_large_tiles(ops, m, n, k):
     """Shapes with at least 256 tiles of 128 x 128 and K a multiple of 64 take the kernel whose slabs go
     straight into LDS: edge tiles in both directions (rows past the end are read from the last valid
-    row and never stored), one slab, an odd number of slabs. The last two have many more rows than
-    columns and tile counts that divide by the XCD grid (2 x 4 with 128-wide tiles, 4 x 2 with 64-wide
-    ones): each XCD then owns a rectangle of tiles, with the matrix's edges in some of them. The two after
-    them take 128 x 192 tiles (32 columns of tiles make one round of blocks, the last one cut off) and
-    128 x 64 tiles; the last three 256 x 256 tiles of eight waves (400 tiles with both edges ragged, exactly
-    one round of 256, few rows of a wide matrix)."""
+    row and never stored), one slab, an odd number of slabs. Which tile shape a product takes follows a
+    time model: with a short K the fixed part decides and most of the first row take 128 x 64 tiles, the
+    fourth and the last of the second row 128 x 128. (4000, 1500) and (1990, 1000) have many more rows
+    than columns and tile counts that divide by the XCD grid: each XCD then owns a rectangle of tiles,
+    with the matrix's edges in some of them. The third row: 128 x 160 tiles (32 columns of tiles, the last
+    one cut off, exactly 512 tiles; and 33 rows of 7 tiles), 128 x 192 tiles (many rows, and few rows of
+    a wide matrix). The last row: 256 x 256 tiles of eight waves (exactly one round of 256 with both edges
+    ragged, and 240 tiles)."""
     x, w = rand((m, k), BF16, 14), rand((n, k), BF16, 15)
     want = x.double() @ w.double().T
     close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
