@@ -95,19 +95,20 @@ def main() -> int:
         say(f"building the {name} shape ({cfg['num_hidden_layers']} of {full} layers, {args.dtype})")
         return cfg, full, random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
 
-    def decode_run(model, cfg, batch, steps, warmup, sampler=None, describe=False):
+    def decode_run(model, cfg, batch, steps, warmup, sampler=None, describe=False, context=None):
         """Decode ``steps`` timed tokens for ``batch`` requests ending at the context length, after the
         warm-up; returns a dict with the rate, the step time and the step's share of the roofline."""
+        context = context or args.context
         warm_steps = max(warmup, math.ceil(args.warmup_seconds / STEP_TIME_FLOOR_S))
         total = warm_steps + steps
-        # Decoding requests keep decoding while later ones are still prefilled (about two steps per
-        # request at a step budget of 2,048 tokens): prompts are shortened by that much, so that the
-        # longest sequence ends at the context length.
-        lead = 2 * batch
-        plen = args.context - total - lead
+        # Decoding requests keep decoding while later ones are still prefilled (a step per 2,048 prompt
+        # tokens of each): prompts are shortened by that much, so that the longest sequence ends at the
+        # context length.
+        lead = batch * max(2, math.ceil((context - total) / 2048))
+        plen = context - total - lead
         if plen < 1:
-            raise SystemExit(f"context {args.context} is too short for {total} decode steps")
-        eng = Engine(model, max_running=batch, kv_pool_tokens=batch * (args.context + 32), chunked_prefill_size=2048,
+            raise SystemExit(f"context {context} is too short for {total} decode steps")
+        eng = Engine(model, max_running=batch, kv_pool_tokens=batch * (context + 32), chunked_prefill_size=2048,
                      decode_graph=not args.no_graph)
         reqs = [eng.add_request(p, SamplingParams(max_new_tokens=total + lead + 8)) for p in prompts(cfg["vocab_size"], batch, plen)]
         say(f"batch {batch}: prefilling {batch} x {plen} tokens")
@@ -277,10 +278,17 @@ def main() -> int:
                                  "decode_frac_of_read": round(achieved / read, 4)}
 
     if not (args.no_points or args.no_extra or args.prefill_only) and args.preset == "0.6B" and not args.layers:
+        points = out["points"]
+        # further context lengths: decode behind 32,768 tokens, a prompt of 8,192 in one step
+        r = decode_run(model, cfg, 8, 24, 8, context=32768)
+        points["decode_b8_ctx32768"] = round(r["tok_s"], 1)
+        points["decode_b8_ctx32768_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
+        p = prefill_run(model, cfg, 8192, 0, repeats=3)
+        points["prefill_8192"] = p["value"]
+        points["prefill_8192_frac"] = p["frac"]
         del model
         gc.collect()
         torch.cuda.empty_cache()
-        points = out["points"]
         cfg8, _, m8 = make("8B")
         for b, steps in ((1, 32), (8, 32), (64, 16)):
             r = decode_run(m8, cfg8, b, steps, 8)
@@ -289,6 +297,12 @@ def main() -> int:
         p8 = prefill_run(m8, cfg8, 2048, 0)
         points["8B_prefill_2048"] = p8["value"]
         points["8B_prefill_2048_frac"] = p8["frac"]
+        r = decode_run(m8, cfg8, 8, 16, 8, context=32768)
+        points["8B_decode_b8_ctx32768"] = round(r["tok_s"], 1)
+        points["8B_decode_b8_ctx32768_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
+        p8 = prefill_run(m8, cfg8, 8192, 0, repeats=3)
+        points["8B_prefill_8192"] = p8["value"]
+        points["8B_prefill_8192_frac"] = p8["frac"]
         del m8
         gc.collect()
         torch.cuda.empty_cache()

@@ -618,7 +618,7 @@ static const TileShape TILE_SHAPES[5] = {
 
 // `pairs`: the gated epilogue needs an even number of 16-column fragments per wave, which 160 columns
 // over two waves are not.
-static int pick_tile_cols(int M, int N, int K, int splits, bool pairs) {
+static int pick_tile_cols(int M, int N, int K, int splits, bool pairs, float* predicted = nullptr) {
   const float slabs = (float)((K + BK - 1) / BK) / splits;
   int best = 128;
   float least = 0.f;
@@ -640,6 +640,7 @@ static int pick_tile_cols(int M, int N, int K, int splits, bool pairs) {
       best = t.cols;
     }
   }
+  if (predicted) *predicted = least;
   return best;
 }
 
@@ -866,12 +867,32 @@ static bool tile_small_matrix(int N, int K) { return (long)N * K * 2 <= (16L << 
 
 extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles >= 256) return 1;
-  if (M > 512) {  // many rows, a narrow matrix: as many splits as fill the chip with 128 x 128 tiles, at most 4
+  if (tiles >= 256 && M <= 512) return 1;
+  if (M > 512 && tiles * 4 < 256) {  // many rows of a narrow matrix: as many splits as fill the chip, at most 4
     int s = (int)((256 + tiles - 1) / tiles);
     if (s > 4) s = 4;
     while (s > 1 && K / s < 512) --s;
     return s;
+  }
+  if (M > 512) {
+    // Up to four splits with at least 16 slabs each, by the time the tile shapes' model predicts plus
+    // what the partial sums cost: each split writes M x N floats and the consumer reads them all, where
+    // one product adds into the residual stream in place (measured about 3.5 TB/s for both).
+    int best = 0;
+    float least = 0.f;
+    for (int sp = 1; sp <= 4; ++sp) {
+      if (tiles * sp < 256 || (sp > 1 && K / sp < 16 * BK)) continue;
+      float t;
+      pick_tile_cols(M, N, K, sp, false, &t);
+      if (sp > 1) t += (float)M * N * 4.f * (2 * sp - 1) / 3.5e6f;
+      if (best == 0 || t < least) {
+        least = t;
+        best = sp;
+      }
+    }
+    if (best == 0) best = tiles >= 256 ? 1 : (int)((256 + tiles - 1) / tiles);
+    const int slabs = (K + BK - 1) / BK, per = (slabs + best - 1) / best;
+    return (slabs + per - 1) / per;  // no empty split
   }
   long want, most;
   if (tile_small_matrix(N, K)) {
