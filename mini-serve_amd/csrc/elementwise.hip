@@ -121,6 +121,20 @@ __device__ __forceinline__ void add_splits(float4& acc, const float* __restrict_
   }
 }
 
+// Four consecutive weights in one load (w + i is aligned to four elements), kept as loaded: what uses
+// them comes after the block's sum, and a conversion right after the load would wait for it there.
+template <typename TW> struct Weights4;
+template <> struct Weights4<float> {
+  float4 v;
+  __device__ __forceinline__ void load(const float* w) { v = *reinterpret_cast<const float4*>(w); }
+  __device__ __forceinline__ float at(int e) const { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
+};
+template <> struct Weights4<bf16> {
+  union { uint2 u; bf16 e[4]; } v;
+  __device__ __forceinline__ void load(const bf16* w) { v.u = *reinterpret_cast<const uint2*>(w); }
+  __device__ __forceinline__ float at(int e) const { return to_f32(v.e[e]); }
+};
+
 template <typename TW, int NT>
 __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x, const TW* __restrict__ w,
                                                             bf16* __restrict__ y, const int* __restrict__ rows, int width,
@@ -132,12 +146,14 @@ __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x,
   float* src = x + row * width;
   const bool in_place = parts != nullptr && rows == nullptr;
   float4 kept[2];
+  Weights4<TW> wk[2];  // asked for with the row: after the block's sum they would cost a second wait
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int i = (threadIdx.x + j * NT) * 4;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < width) {
+      wk[j].load(w + i);
       v = *reinterpret_cast<const float4*>(src + i);
       if (parts != nullptr) {
         const float* p = parts + row * width + i;
@@ -166,10 +182,10 @@ __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x,
     const int i = (threadIdx.x + j * NT) * 4;
     if (i < width) {
       union { uint2 u; bf16 e[4]; } o;
-      o.e[0] = from_f32<bf16>(kept[j].x * rstd * to_f32(w[i]));
-      o.e[1] = from_f32<bf16>(kept[j].y * rstd * to_f32(w[i + 1]));
-      o.e[2] = from_f32<bf16>(kept[j].z * rstd * to_f32(w[i + 2]));
-      o.e[3] = from_f32<bf16>(kept[j].w * rstd * to_f32(w[i + 3]));
+      o.e[0] = from_f32<bf16>(kept[j].x * rstd * wk[j].at(0));
+      o.e[1] = from_f32<bf16>(kept[j].y * rstd * wk[j].at(1));
+      o.e[2] = from_f32<bf16>(kept[j].z * rstd * wk[j].at(2));
+      o.e[3] = from_f32<bf16>(kept[j].w * rstd * wk[j].at(3));
       *reinterpret_cast<uint2*>(dst + i) = o.u;
     }
   }
