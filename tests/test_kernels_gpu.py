@@ -253,8 +253,11 @@ def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 8), (2048, 1024, 3072, 2), (300, 1000, 1100, 6), (2048, 4096, 1024, 1),
-                                          (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6)])
+                                          (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6),
+                                          (1024, 4096, 12288, 2), (768, 5120, 8192, 2)])
 def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
+    """The last two have 256 and more tiles of 128 x 128 already: above 512 rows the splits follow the
+    predicted time (a long K in two halves fills two blocks per CU), not the tile count alone."""
     x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
     want = x.double() @ w.double().T
     resid = rand((m, n), F32, 62)
