@@ -270,11 +270,14 @@ def main() -> int:
         buf = torch.empty((n,), dtype=torch.uint8, device="cuda:0").random_(0, 256)
         read = n / median_ms(lambda: ops.measure_read(buf)) / 1e6
         del buf
-        x = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
-        w = torch.randn((4096, 4096), device="cuda:0").to(torch.bfloat16)
-        rate = 2 * 4096**3 / median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16)) / 1e9
-        del x, w
-        out["measured_peaks"] = {"read_GBps": round(read, 1), "gemm_bf16_4096_TFLOPs": round(rate, 1),
+        rates = {}
+        for n in (4096, 8192):
+            x = torch.randn((n, n), device="cuda:0").to(torch.bfloat16)
+            w = torch.randn((n, n), device="cuda:0").to(torch.bfloat16)
+            rates[n] = 2 * n**3 / median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16)) / 1e9
+            del x, w
+        out["measured_peaks"] = {"read_GBps": round(read, 1), "gemm_bf16_4096_TFLOPs": round(rates[4096], 1),
+                                 "gemm_bf16_8192_TFLOPs": round(rates[8192], 1),
                                  "decode_frac_of_read": round(achieved / read, 4)}
 
     if not (args.no_points or args.no_extra or args.prefill_only) and args.preset == "0.6B" and not args.layers:

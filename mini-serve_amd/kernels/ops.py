@@ -119,6 +119,14 @@ def _check(code: int, what: str) -> None:
 
 
 def _dev(t: torch.Tensor, name: str, dtypes, ndim: int | None = None) -> None:
+    """A contiguous tensor on the GPU of one of ``dtypes`` (and of ``ndim`` dimensions). A model pass
+    makes hundreds of these checks: what is right passes in three calls; what is wrong is looked at
+    again, slowly, for the message."""
+    try:
+        if t.is_cuda and t.is_contiguous() and (t.dtype is dtypes or t.dtype in dtypes) and (ndim is None or t.dim() == ndim):
+            return
+    except (AttributeError, TypeError):
+        pass
     if not isinstance(t, torch.Tensor) or not t.is_cuda:
         raise TypeError(f"{name} must be a tensor on the GPU")
     if t.dtype not in (dtypes if isinstance(dtypes, tuple) else (dtypes,)):
