@@ -253,8 +253,9 @@ def main() -> int:
         # What this box gives beside the published peaks (the same kernels as `python -m miniserve_amd roofline`).
         from miniserve_amd.kernels import ops
 
-        def median_ms(fn, repeats=5):
-            fn()
+        def median_ms(fn, repeats=9, warm=3):
+            for _ in range(warm):
+                fn()
             torch.cuda.synchronize()
             times = []
             for _ in range(repeats):
