@@ -238,6 +238,34 @@ def test_nucleus_keeps_the_smallest_set_reaching_top_p():
     assert {P.sample(tie, 1.0, s, 0, top_p=0.3) for s in range(300)} == {0, 1}  # ties stay in index order
 
 
+def test_nucleus_on_the_vectors_of_the_reference_s_sampler_tests():
+    """The cases of the reference's tests/test_sampler.py:73-96, with its own numbers: the mass before
+    each token of (0.4, 0.3, 0.2, 0.06, 0.04) is 0, 0.4, 0.7, 0.9, 0.96, so top_p 0.8 keeps three and draws
+    them in their renormalised shares; a tiny top_p leaves the most likely token whatever the
+    temperature; the nucleus goes by probability, not by token id."""
+    probs = np.array([0.4, 0.3, 0.2, 0.06, 0.04])
+    draws = [P.sample(np.log(probs), 1.0, seed, 0, top_p=0.8) for seed in range(6000)]
+    freq = np.bincount(draws, minlength=5) / 6000
+    assert freq[3] == 0 and freq[4] == 0
+    assert np.abs(freq[:3] - probs[:3] / probs[:3].sum()).max() < 0.025
+    assert {P.sample(np.array([0.1, 2.0, 1.9, -1.0]), 3.0, seed, 0, top_p=1e-6) for seed in range(500)} == {1}
+    shuffled = np.array([0.04, 0.2, 0.06, 0.4, 0.3])
+    seen = np.bincount([P.sample(np.log(shuffled), 1.0, seed, 0, top_p=0.8) for seed in range(3000)], minlength=5)
+    assert seen[0] == 0 and seen[2] == 0 and (seen[[1, 3, 4]] > 0).all()
+
+
+def test_a_draw_depends_on_its_seed_and_position_alone():
+    """tests/test_sampler.py:101-113 of the reference: a row's sample is a function of (seed, counter,
+    logits); here also of nothing else in the call (the vocabulary's other rows do not exist for it)."""
+    r = np.random.default_rng(1)
+    for trial in range(20):
+        row = r.standard_normal(1000)
+        a = P.sample(row, 1.0, 1000 + trial, trial, top_p=0.9)
+        assert a == P.sample(row.copy(), 1.0, 1000 + trial, trial, top_p=0.9)
+        others = {P.sample(row, 1.0, 1000 + trial, trial + k, top_p=0.9) for k in range(1, 40)}
+        assert len(others) > 1  # another position draws other noise
+
+
 # ------------------------------------------------------------------------------------------ wiring of a layer
 #
 # What the part tests above cannot see: which norm feeds which product, where the per-head norms sit
