@@ -121,6 +121,57 @@ def test_read_back_one_step_behind_changes_nothing(folders, dtype, graph):
         assert outs[True][i][:6] == want
 
 
+def test_a_step_returns_without_waiting_for_what_it_launches(folders):
+    """With the read-back one step behind, ``step`` launches a batch and reads the tokens of the batch
+    before it: it must not wait for the device to reach the new one. A long piece of device work is
+    queued between two steps; the second step's own batch lies behind it, the batch it reads back ran
+    before it, so the step returns long before that work ends. Without the overlap (the control: the
+    measurement could not fail if this did not wait) the step reads its own batch back and takes as long
+    as the queued work. Decode steps replayed from a graph and steps launched kernel by kernel alike."""
+    import time
+
+    import torch
+
+    from miniserve_amd.engine.request import RequestState, SamplingParams
+
+    cfg, _ = read_model_folder(folders["tinyB"])
+    big = torch.randn((8192, 8192), device="cuda:0").to(torch.bfloat16)
+
+    def busy():
+        for _ in range(48):
+            torch.matmul(big, big)
+
+    busy()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    busy()
+    torch.cuda.synchronize()
+    busy_s = time.perf_counter() - t
+    assert busy_s > 0.02, "the queued work is too short to measure against"
+    for overlap, graph in ((True, True), (True, False), (False, True)):
+        eng = engine(folders["tinyB"], "bfloat16", kv_pool_tokens=2048, max_running=4, decode_graph=graph, overlap=overlap)
+        reqs = [eng.add_request(p, SamplingParams(max_new_tokens=60)) for p in prompts_for(cfg, [20, 33, 9, 41], seed=4)]
+        while any(r.state is not RequestState.DECODE for r in reqs):
+            eng.step()
+        for _ in range(3):
+            eng.step()
+        torch.cuda.synchronize()
+        eng.step()
+        busy()
+        t = time.perf_counter()
+        eng.step()
+        elapsed = time.perf_counter() - t
+        torch.cuda.synchronize()
+        if overlap:
+            assert elapsed < 0.25 * busy_s, f"step took {elapsed * 1e3:.1f} ms with {busy_s * 1e3:.0f} ms of work queued ahead of its batch"
+            assert not graph or eng.runner.graph_steps > 0
+        else:
+            assert elapsed > 0.8 * busy_s, f"the control did not wait: {elapsed * 1e3:.1f} ms of {busy_s * 1e3:.0f}"
+        while eng.has_unfinished:
+            eng.step()
+        assert eng.runner.cache.idle
+
+
 def test_sampled_requests_reproduce_beside_greedy_ones(folders):
     """Temperature sampling with a request seed: the same tokens alone, in a batch, and after
     preemption; equal to the plain sampler run on the plain logits."""
