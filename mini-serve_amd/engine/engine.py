@@ -143,6 +143,8 @@ class Engine:
         self.launched = batch
         launched = self._launch(batch, prev) if batch is not None else None
         if not self.overlap:
+            if prev is not None:  # ``overlap`` was switched off between two steps: the step before is still due
+                self._finish(prev)
             return self._finish(launched) if launched is not None else None
         self._inflight = launched
         return self._finish(prev) if prev is not None else None

@@ -167,9 +167,10 @@ def test_a_step_returns_without_waiting_for_what_it_launches(folders):
             assert not graph or eng.runner.graph_steps > 0
         else:
             assert elapsed > 0.8 * busy_s, f"the control did not wait: {elapsed * 1e3:.1f} ms of {busy_s * 1e3:.0f}"
+        eng.overlap = not overlap  # switched between two steps: no token is lost or read twice
         while eng.has_unfinished:
             eng.step()
-        assert eng.runner.cache.idle
+        assert eng.runner.cache.idle and all(len(r.output_ids) == 60 and r.in_flight == 0 for r in reqs)
 
 
 def test_sampled_requests_reproduce_beside_greedy_ones(folders):
