@@ -14,8 +14,9 @@ what the GPU's clock did meanwhile is in ``sidecar``).
 One JSON line is printed. ``value`` = decoded tokens per second of the headline point. Beside it:
 ``prefill`` (one 2,048-token prompt in one step; median of five), ``roofline`` (the decode step's bytes,
 every weight once plus the live requests' cache, over its time, against the published 8 TB/s),
-``points`` (decode at batch 1 and 64 of the same shape; with ``--extra``, on by default, the Qwen3-8B
-shape's decode at batch 1 / 8 / 64 and prefill, and the Qwen3-32B shape's continuous batching of 64
+``points`` (decode at batch 1 and 64 of the same shape; unless ``--no-extra``, decode at batch 8 behind
+32,768 tokens and a prompt of 8,192 tokens in one step, the Qwen3-8B shape's decode at batch 1 / 8 / 64, its
+prefill and the same two further lengths, and the Qwen3-32B shape's continuous batching of 64
 requests with 2,048-token prompts under a 512-token step budget, decode-only and mixed steps timed
 apart, each with its share of the roofline), ``measured_peaks`` (what this box gives a streaming read
 and the engine's bfloat16 product) and ``sidecar`` (device, clocks and power while the headline point
