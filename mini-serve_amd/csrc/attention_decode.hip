@@ -155,17 +155,26 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
   const bool has_new = FUSED && fin.store && w_begin < w_end && w_end == n_chunks;
   __shared__ __attribute__((aligned(16))) bf16 qs[FUSED ? 4 : 1][FUSED ? 16 * D : 8];  // each wave's queries [G, D]
   __shared__ __attribute__((aligned(16))) bf16 kv_new[FUSED ? 2 * D : 8];              // the new key, then the new value
+  // The two table entries of a chunk are fetched together and without a condition (one 8-byte load where
+  // the table allows it; past the wave's last chunk that chunk's again, dropped): a load that waits for
+  // the outcome of another costs a round trip each, before the first key is even asked for. Whether the
+  // chunk has a second page at all is settled when the entries are used.
+  const bool pair_ids = (table_width % 2 == 0) && (reinterpret_cast<size_t>(block_table) % 8 == 0);
   int p0n = 0, p1n = 0;
   auto fetch_ids = [&](int c) {
-    if (c < w_end) {
-      const int t0 = lo_al + c * CHUNK;
-      p0n = table[t0 / PAGE];
-      p1n = (t0 + PAGE < kv_len) ? table[t0 / PAGE + 1] : p0n;
+    const int idx = (lo_al + min(c, w_end - 1) * CHUNK) / PAGE;  // even: a chunk is two pages
+    if (pair_ids) {
+      const int2 v = *reinterpret_cast<const int2*>(table + idx);
+      p0n = v.x;
+      p1n = v.y;
+    } else {
+      p0n = table[idx];
+      p1n = table[min(idx + 1, table_width - 1)];
     }
   };
   auto load = [&](DecodeTile<D>& t, int c) {
     const int p0 = max(p0n, 0);  // a page behind the window was given back: its tokens are masked below
-    const int p1 = max(p1n, 0);
+    const int p1 = (lo_al + c * CHUNK + PAGE < kv_len) ? max(p1n, 0) : p0;
     fetch_ids(c + 1);
     // Key rows: lane r feeds row r of both products. Product a takes tokens 0-3 and 8-11 of each page,
     // product b tokens 4-7 and 12-15 (rows 0-7 from the chunk's first page, 8-15 from its second).
@@ -254,8 +263,10 @@ __global__ __launch_bounds__(256, 2) void attn_decode_split_kernel(
   {
     DecodeTile<D> ta, tb;
     int c = w_begin;
-    fetch_ids(c);
-    if (c < w_end) load(ta, c);
+    if (c < w_end) {
+      fetch_ids(c);
+      load(ta, c);
+    }
     if (FUSED) {
       // Queries of the group: G * D floats, four per lane and round. (The first chunk is on its way.)
       const size_t row = (size_t)tok * fin.row_width;
