@@ -76,4 +76,13 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ p, int spl
   return acc;
 }
 
+// Activations of the gated feed-forward, by the number the host passes: out = act(gate) * up, in float32.
+#define MS_ACT_SILU 0
+#define MS_ACT_GELU_TANH 1
+#define MS_ACT_COUNT 2
+__device__ __forceinline__ float activate(float x, int act) {
+  if (act == MS_ACT_GELU_TANH) return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+  return x / (1.f + expf(-x));
+}
+
 static inline int launch_status() { return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED; }

@@ -226,7 +226,7 @@ extern "C" int ms_rmsnorm(float* x, const void* w, int w_is_bf16, void* y, int y
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t, i] = silu(gate[t, i]) * up[t, i] for a row gu[t] that holds both, in one of two layouts:
+// out[t, i] = act(gate[t, i]) * up[t, i] (act: an MS_ACT_* number) for a row gu[t] that holds both, in one of two layouts:
 //   block == 0: the gates, then the ups:                 gate i at i, up i at inter + i
 //   block  > 0: alternating runs of `block` gates and `block` ups (the order a matrix product over
 //               interleaved weight rows leaves them in): gate i at (i / block) * 2 block + i % block,
@@ -235,30 +235,30 @@ __device__ __forceinline__ int gate_at(int i, int block) { return block ? (i / b
 __device__ __forceinline__ int up_at(int i, int inter, int block) { return block ? gate_at(i, block) + block : inter + i; }
 
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int block) {
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int block, int act) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const float g = to_f32(gu[(size_t)t * 2 * inter + gate_at(i, block)]);
   const float u = to_f32(gu[(size_t)t * 2 * inter + up_at(i, inter, block)]);
-  out[(size_t)t * inter + i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  out[(size_t)t * inter + i] = from_f32<T>(activate(g, act) * u);
 }
 
 // The same with gu given as float partial sums [splits, tokens, 2 * inter] (summed in ascending order).
 template <typename T>
-__global__ void silu_mul_parts_kernel(const float* __restrict__ parts, int splits, size_t split_stride,
-                                      T* __restrict__ out, int inter, int block) {
+__global__ void act_mul_parts_kernel(const float* __restrict__ parts, int splits, size_t split_stride,
+                                     T* __restrict__ out, int inter, int block, int act) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const float* row = parts + (size_t)t * 2 * inter;
   const float g = sum_splits(row + gate_at(i, block), splits, split_stride);
   const float u = sum_splits(row + up_at(i, inter, block), splits, split_stride);
-  out[(size_t)t * inter + i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  out[(size_t)t * inter + i] = from_f32<T>(activate(g, act) * u);
 }
 
 // bfloat16 with inter (and block) a multiple of 8: eight elements per thread, moved as 16-byte vectors.
-__global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int inter, int block) {
+__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int inter, int block, int act) {
   const int t = blockIdx.y;
   const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (i >= inter) return;
@@ -268,29 +268,30 @@ __global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restri
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float gv = to_f32(g.e[e]);
-    o.e[e] = from_f32<bf16>(gv / (1.f + expf(-gv)) * to_f32(u.e[e]));
+    o.e[e] = from_f32<bf16>(activate(gv, act) * to_f32(u.e[e]));
   }
   *reinterpret_cast<uint4*>(out + (size_t)t * inter + i) = o.u;
 }
 
-extern "C" int ms_silu_mul(const void* gu, void* out, int is_bf16, int tokens, int inter, int block, hipStream_t st) {
+extern "C" int ms_act_mul(const void* gu, void* out, int is_bf16, int tokens, int inter, int block, int act, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (inter <= 0 || tokens > 65535 || block < 0 || (block > 0 && inter % block)) return MS_BAD_ARG;
+  if (inter <= 0 || tokens > 65535 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_ACT_COUNT) return MS_BAD_ARG;
   dim3 grid((inter + 255) / 256, tokens);
   if (is_bf16 && inter % 8 == 0 && block % 8 == 0)
-    silu_mul_vec8_kernel<<<dim3((inter / 8 + 255) / 256, tokens), 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block);
-  else if (is_bf16) silu_mul_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block);
-  else silu_mul_kernel<float><<<grid, 256, 0, st>>>((const float*)gu, (float*)out, inter, block);
+    act_mul_vec8_kernel<<<dim3((inter / 8 + 255) / 256, tokens), 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act);
+  else if (is_bf16) act_mul_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act);
+  else act_mul_kernel<float><<<grid, 256, 0, st>>>((const float*)gu, (float*)out, inter, block, act);
   return launch_status();
 }
 
-extern "C" int ms_silu_mul_parts(const float* parts, int splits, long long split_stride, void* out, int out_is_bf16,
-                                 int tokens, int inter, int block, hipStream_t st) {
+extern "C" int ms_act_mul_parts(const float* parts, int splits, long long split_stride, void* out, int out_is_bf16,
+                                int tokens, int inter, int block, int act, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (inter <= 0 || tokens > 65535 || splits < 1 || block < 0 || (block > 0 && inter % block)) return MS_BAD_ARG;
+  if (inter <= 0 || tokens > 65535 || splits < 1 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_ACT_COUNT)
+    return MS_BAD_ARG;
   dim3 grid((inter + 255) / 256, tokens);
-  if (out_is_bf16) silu_mul_parts_kernel<bf16><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (bf16*)out, inter, block);
-  else silu_mul_parts_kernel<float><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (float*)out, inter, block);
+  if (out_is_bf16) act_mul_parts_kernel<bf16><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (bf16*)out, inter, block, act);
+  else act_mul_parts_kernel<float><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (float*)out, inter, block, act);
   return launch_status();
 }
 

@@ -340,9 +340,9 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
         for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
   }
 
-  if (mode == 3) {
-    // Gated epilogue: W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and
-    // 2 p + 1 of a lane are gate and up of the same four outputs: out[m, n / 2 ...] = silu(gate) * up,
+  if (mode >= 3) {
+    // Gated epilogue (mode 3 + an MS_ACT_* number): W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and
+    // 2 p + 1 of a lane are gate and up of the same four outputs: out[m, n / 2 ...] = act(gate) * up,
     // bf16 [M, N / 2] with row stride ldc. Wave tiles with an odd number of fragments are never
     // launched in this mode.
 #pragma unroll
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float gate = acc[i][j][e];
-            o.e[e] = static_cast<bf16>(gate / (1.f + expf(-gate)) * acc[i + 1][j][e]);
+            o.e[e] = static_cast<bf16>(activate(gate, mode - 3) * acc[i + 1][j][e]);
           }
           *reinterpret_cast<uint2*>((bf16*)Cbase + (size_t)m * ldc + col) = o.u;
         }
@@ -742,7 +742,7 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Gated feed-forward input for few rows (M <= 16 MB): out[m, i] = silu(x . gate_i) * (x . up_i), bf16
+// Gated feed-forward input for few rows (M <= 16 MB): out[m, i] = act(x . gate_i) * (x . up_i), bf16
 // [M, inter], from W [2 inter, K] that holds alternating blocks of 16 gate rows and 16 up rows. One
 // block of 8 waves per 16 outputs: waves 0-3 take the gate rows, waves 4-7 the up rows, wave w of each
 // four the K slabs w, w + 4, ... (one slab each up to K = 1024: all loads of the block in flight at
@@ -750,7 +750,9 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
 // comes from the cache). The eight partial results meet in LDS; wave i % 8 adds those of rows 16 i ..
 // in wave order, applies the activation and stores. No partial sums leave the block and no second
 // kernel runs. K must be a multiple of 256 and rows 16-byte aligned.
-template <int MB>
+// (ACT is a template parameter here: the kernel is a chain of latencies, and the choice inside it measured 0.6 % of
+// a decode step of one row.)
+template <int MB, int ACT>
 __global__ __launch_bounds__(512) void gemm_bf16_small_gated_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                     bf16* __restrict__ out, int M, int inter, int K,
                                                                     int ldx) {
@@ -808,27 +810,30 @@ __global__ __launch_bounds__(512) void gemm_bf16_small_gated_kernel(const bf16* 
         gate += red[w][i][lane][e];
         up += red[4 + w][i][lane][e];
       }
-      o.e[e] = static_cast<bf16>(gate / (1.f + expf(-gate)) * up);
+      o.e[e] = static_cast<bf16>(activate(gate, ACT) * up);
     }
     *reinterpret_cast<uint2*>(out + (size_t)m * inter + blockIdx.x * 16 + g * 4) = o.u;
   }
 }
 
-// out bf16 [M, inter] = silu(X gate^T) * (X up^T) for W [2 inter, K] with gate and up rows in
+// out bf16 [M, inter] = act(X gate^T) * (X up^T) (act: an MS_ACT_* number) for W [2 inter, K] with gate and up rows in
 // alternating blocks of 16. MS_UNSUPPORTED for shapes no fused kernel takes (the caller then runs the
 // product and the activation separately): K no multiple of 64 (of 256 for M <= 64) or unaligned rows,
 // more K than a block of the small kernel should walk alone (2048 up to 16 rows, 1024 up to 32), 33 to
 // 64 rows of a large matrix (those stream the weights with K split over blocks).
-extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M, int inter, int K, int ldx, hipStream_t st) {
+extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M, int inter, int K, int ldx, int act,
+                                  hipStream_t st) {
   if (M <= 0 || inter <= 0) return MS_OK;
-  if (K <= 0 || ldx < K) return MS_BAD_ARG;
+  if (K <= 0 || ldx < K || act < 0 || act >= MS_ACT_COUNT) return MS_BAD_ARG;
+  const int gated = 3 + act;  // the tile kernel's mode
   if (inter % 16 || ldx % 8) return MS_UNSUPPORTED;
   const bf16* x = (const bf16*)X;
   const bf16* w = (const bf16*)W;
   const int N = 2 * inter;
   if (M <= 16) {
     if (K % SMALL_SLAB || K / SMALL_SLAB > 8) return MS_UNSUPPORTED;
-    gemm_bf16_small_gated_kernel<1><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    if (act == MS_ACT_SILU) gemm_bf16_small_gated_kernel<1, MS_ACT_SILU><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    else gemm_bf16_small_gated_kernel<1, MS_ACT_GELU_TANH><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
     return launch_status();
   }
   if (M <= 32 && K % SMALL_SLAB == 0 && K / SMALL_SLAB <= 4) {
@@ -836,7 +841,8 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
     // slabs covers K (each wave then holds its slab of every row at once): 7.8 against 9.2 us at the
     // 0.6B shape. Larger K streams the weights with K split over blocks and runs the activation as a
     // kernel of its own.
-    gemm_bf16_small_gated_kernel<2><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    if (act == MS_ACT_SILU) gemm_bf16_small_gated_kernel<2, MS_ACT_SILU><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
+    else gemm_bf16_small_gated_kernel<2, MS_ACT_GELU_TANH><<<inter / 16, 512, 0, st>>>(x, w, (bf16*)out, M, inter, K, ldx);
     return launch_status();
   }
   if (K % BK) return MS_UNSUPPORTED;
@@ -844,14 +850,14 @@ extern "C" int ms_gemm_bf16_gated(const void* X, const void* W, void* out, int M
     // 33 to 64 rows (one row of 64 x 64 tiles): the tile kernel with the activation in its epilogue
     // where the matrix is small enough that K need not be split to keep the chip busy.
     if (M > 32 && (long)N * K * 2 <= (16L << 20) && (N + 63) / 64 >= 96)
-      return launch_dma<64, 64, BK, 2, 4>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+      return launch_dma<64, 64, BK, 2, 4>(x, w, out, gated, M, N, K, ldx, inter, K, 0, 1, st);
     return MS_UNSUPPORTED;
   }
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (big >= 256) return launch_picked(pick_tile_cols(M, N, K, 1, true), x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  if (big >= 256) return launch_picked(pick_tile_cols(M, N, K, 1, true), x, w, out, gated, M, N, K, ldx, inter, K, 0, 1, st);
   // 64 x 64 tiles from 128 of them on: half the CUs without a split of K still beat the split product
   // followed by the activation kernel (10.2 against 11.8 to 13.1 us at 65 to 128 rows of the 0.6B shape).
-  if ((long)((M + 63) / 64) * ((N + 63) / 64) >= 128) return launch_dma<64, 64, BK, 2, 4>(x, w, out, 3, M, N, K, ldx, inter, K, 0, 1, st);
+  if ((long)((M + 63) / 64) * ((N + 63) / 64) >= 128) return launch_dma<64, 64, BK, 2, 4>(x, w, out, gated, M, N, K, ldx, inter, K, 0, 1, st);
   return MS_UNSUPPORTED;  // too few tiles without a split of K
 }
 

@@ -24,9 +24,9 @@ _SIGNATURES = {
     "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
     "ms_feed_tokens": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int, _c_ll, _c_void],
-    "ms_silu_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_silu_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_act_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_act_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
     "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
@@ -243,12 +243,23 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return both.reshape(2 * i, k).contiguous()
 
 
+# Activations of the gated feed-forward and the numbers the kernels know them by (MS_ACT_* in csrc/common.h):
+# silu(x) = x sigmoid(x); gelu_tanh(x) = x / 2 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))).
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def _activation(name: str) -> int:
+    try:
+        return ACTIVATIONS[name]
+    except KeyError:
+        raise NotImplementedError(f"activation {name!r}: the kernels know {sorted(ACTIVATIONS)}") from None
+
+
 def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> torch.Tensor:
     """``act(gate) * up`` for ``gu [T, 2 I]``, a tensor or a ``SplitSum`` (then ``out_dtype`` names the
     result's dtype). ``block == 0``: the row holds the ``I`` gates, then the ``I`` ups; ``block > 0``:
     alternating runs of ``block`` gates and ``block`` ups (see ``interleave_gate_up``)."""
-    if activation != "silu":
-        raise NotImplementedError(f"activation {activation!r}")
+    act = _activation(activation)
     if isinstance(gu, SplitSum):
         _dev(gu.parts, "gu", F32, 3)
         t, width = gu.shape
@@ -257,8 +268,8 @@ def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> tor
         out = torch.empty((t, width // 2), dtype=out_dtype, device=gu.parts.device)
         for t0 in range(0, t, 32768):
             n = min(32768, t - t0)
-            _check(library().ms_silu_mul_parts(gu.parts[:, t0:].data_ptr(), gu.splits, gu.stride, out[t0:].data_ptr(),
-                                               int(out_dtype == BF16), n, width // 2, int(block), _stream()), "silu_mul")
+            _check(library().ms_act_mul_parts(gu.parts[:, t0:].data_ptr(), gu.splits, gu.stride, out[t0:].data_ptr(),
+                                              int(out_dtype == BF16), n, width // 2, int(block), act, _stream()), "act_mul")
         return out
     _dev(gu, "gu", (F32, BF16), 2)
     if gu.shape[1] % 2 or (block and (gu.shape[1] // 2) % block):
@@ -268,8 +279,8 @@ def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> tor
     # grid.y carries the token index: split very long batches
     for t0 in range(0, gu.shape[0], 32768):
         n = min(32768, gu.shape[0] - t0)
-        _check(library().ms_silu_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, int(block),
-                                     _stream()), "silu_mul")
+        _check(library().ms_act_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, int(block), act,
+                                    _stream()), "act_mul")
     return out
 
 
@@ -278,8 +289,7 @@ def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu
     interleaved bfloat16 weights the activation runs in the matrix kernel's epilogue where a kernel
     for the shape exists (few rows: no partial sums leave the kernel; many rows: the gate/up matrix is
     never written); otherwise the product and the activation are two kernels."""
-    if activation != "silu":
-        raise NotImplementedError(f"activation {activation!r}")
+    act = _activation(activation)
     _dev(x, "x", (F32, BF16), 2)
     _dev(gate_up, "gate_up", (F32, BF16), 2)
     m, k = x.shape
@@ -289,7 +299,7 @@ def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu
     if block == GATE_BLOCK and gate_up.dtype == BF16 and out_dtype == BF16 and m > 0:
         xa = cast(x, BF16)
         out = torch.empty((m, inter), dtype=BF16, device=x.device)
-        rc = library().ms_gemm_bf16_gated(xa.data_ptr(), gate_up.data_ptr(), out.data_ptr(), m, inter, k, k, _stream())
+        rc = library().ms_gemm_bf16_gated(xa.data_ptr(), gate_up.data_ptr(), out.data_ptr(), m, inter, k, k, act, _stream())
         if rc == 0:
             return out
         if rc != 2:  # 2: no fused kernel for this shape

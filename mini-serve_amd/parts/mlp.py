@@ -13,9 +13,6 @@ from ..config.spec import PartSpec
 from .base import FeedForward, TensorSpec
 from .registry import register
 
-ACTIVATIONS = ("silu",)
-
-
 @register("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
     def __init__(self, spec: PartSpec, rt):
@@ -24,8 +21,8 @@ class GatedMLP(FeedForward):
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
         self.activation = spec.get("activation", "silu")
-        if self.activation not in ACTIVATIONS:
-            raise NotImplementedError(f"activation {self.activation!r} is not supported, expected {ACTIVATIONS}")
+        if self.activation not in rt.ops.ACTIVATIONS:
+            raise NotImplementedError(f"activation {self.activation!r} is not supported, expected one of {sorted(rt.ops.ACTIVATIONS)}")
         self.gate_up = self.down = None
         self.block = 0  # rows per run of gate / up rows in gate_up (0: all gates, then all ups)
 

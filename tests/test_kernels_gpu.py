@@ -4,6 +4,7 @@ in steps of 16, odd head counts and groups, rows that do not fill a tile."""
 
 from __future__ import annotations
 
+import math
 
 import numpy as np
 import pytest
@@ -91,20 +92,40 @@ def test_rmsnorm_eps_enters(ops):
     assert (a - b).abs().max() > 1e-2  # at this scale eps is of the size of mean(x^2)
 
 
+def activation(name, g):
+    """The gate's activation in float64, from its definition: silu(x) = x sigmoid(x); gelu_tanh is the
+    tanh approximation of x Phi(x), x / 2 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))."""
+    if name == "silu":
+        return g / (1 + torch.exp(-g))
+    assert name == "gelu_tanh"
+    return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g**3)))
+
+
+def test_the_two_activations_are_not_each_other():
+    g = torch.linspace(-6, 6, 49, dtype=torch.float64)
+    phi = 0.5 * (1 + torch.erf(g / math.sqrt(2)))
+    assert float((activation("gelu_tanh", g) - g * phi).abs().max()) < 5e-4  # the approximation of x Phi(x)
+    assert float((activation("silu", g) - g * torch.sigmoid(g)).abs().max()) < 1e-15
+    assert float((activation("silu", g) - activation("gelu_tanh", g)).abs().max()) > 0.1
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("inter", [224, 100, 3072])  # a multiple of 8 moves vectors, others single elements
-def test_silu_mul(ops, dtype, inter):
+def test_act_mul(ops, dtype, inter, act):
     gu = rand((5, 2 * inter), dtype, 5, 2.0)
     g, u = gu[:, :inter].double(), gu[:, inter:].double()
-    want = g / (1 + torch.exp(-g)) * u
-    close(ops.act_mul(gu), want, 1e-6 if dtype == F32 else 5e-3, "silu_mul")
+    want = activation(act, g) * u
+    close(ops.act_mul(gu, act), want, 1e-6 if dtype == F32 else 5e-3, "act_mul")
     z = torch.zeros((1, 8), dtype=dtype, device=DEV)
-    assert float(ops.act_mul(z).abs().max()) == 0.0
+    assert float(ops.act_mul(z, act).abs().max()) == 0.0
     if inter % 16 == 0:  # the same values with gates and ups in alternating runs of 16
         mixed = torch.stack((gu[:, :inter].reshape(5, inter // 16, 16), gu[:, inter:].reshape(5, inter // 16, 16)), dim=2)
-        close(ops.act_mul(mixed.reshape(5, 2 * inter).contiguous(), block=16), want, 1e-6 if dtype == F32 else 5e-3, "runs of 16")
+        close(ops.act_mul(mixed.reshape(5, 2 * inter).contiguous(), act, block=16), want, 1e-6 if dtype == F32 else 5e-3, "runs of 16")
         parts = torch.stack([mixed.reshape(5, 2 * inter).float() * f for f in (0.5, 0.25, 0.25)])
-        close(ops.act_mul(ops.SplitSum(parts), out_dtype=dtype, block=16), want, 1e-6 if dtype == F32 else 5e-3, "partial sums")
+        close(ops.act_mul(ops.SplitSum(parts), act, out_dtype=dtype, block=16), want, 1e-6 if dtype == F32 else 5e-3, "partial sums")
+    with pytest.raises(NotImplementedError, match="gelu_tanh"):  # the message names what there is
+        ops.act_mul(gu, "relu")
 
 
 # (rows, width of x, outputs): up to 64 rows run one fused kernel whose waves split K and meet in LDS
@@ -116,20 +137,21 @@ GATED = [(3000, 128, 4096), (1, 1024, 3072), (8, 1024, 3072), (16, 512, 64), (5,
          (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096)]
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("m,k,inter", GATED)
-def test_gated_linear(ops, dtype, m, k, inter):
+def test_gated_linear(ops, dtype, m, k, inter, act):
     x = rand((m, k), dtype, 70)
     gate, up = rand((inter, k), dtype, 71, 0.05), rand((inter, k), dtype, 72, 0.05)
     g, u = x.double() @ gate.double().T, x.double() @ up.double().T
-    want = g / (1 + torch.exp(-g)) * u
+    want = activation(act, g) * u
     w = ops.interleave_gate_up(gate, up)
     assert w.shape == (2 * inter, k) and torch.equal(w[:16], gate[:16]) and torch.equal(w[16:32], up[:16])
-    got = ops.gated_linear(x, w, out_dtype=dtype, block=ops.GATE_BLOCK)
+    got = ops.gated_linear(x, w, act, out_dtype=dtype, block=ops.GATE_BLOCK)
     assert got.shape == (m, inter) and got.dtype == dtype
     close(got, want, 1e-5 if dtype == F32 else 8e-3, f"gated {m}x{k}->{inter}")
     # and with the plain layout (gates, then ups) through the two-kernel path
-    close(ops.gated_linear(x, torch.cat((gate, up)).contiguous(), out_dtype=dtype), want, 1e-5 if dtype == F32 else 8e-3, "halves")
+    close(ops.gated_linear(x, torch.cat((gate, up)).contiguous(), act, out_dtype=dtype), want, 1e-5 if dtype == F32 else 8e-3, "halves")
 
 
 # ------------------------------------------------------------------------------------------ matrix products
@@ -226,7 +248,7 @@ def test_pending_sums_feed_their_consumers(ops, m):
     # gated activation
     gu = ops.linear(x, w, out_dtype=BF16, defer=True)
     g, u = want[:, : n // 2], want[:, n // 2 :]
-    close(ops.act_mul(gu, out_dtype=BF16), g / (1 + torch.exp(-g)) * u, 6e-3, "act_mul of partial sums")
+    close(ops.act_mul(gu, out_dtype=BF16), activation("silu", g) * u, 6e-3, "act_mul of partial sums")
     # without defer the same call returns the finished matrix / adds it
     close(ops.linear(x, w, out_dtype=F32), want, 1e-5, "finished matrix")
     r4 = resid.clone()

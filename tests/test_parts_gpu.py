@@ -76,6 +76,16 @@ def test_feed_forward_alone(dtype):
     with pytest.raises(NotImplementedError):
         bad = PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8, "activation": "gelu"})
         part_class("feed_forward", bad)(bad, rt)
+    # the activation is a parameter of the part, not of the architecture: the other one the kernels know
+    other = PartSpec("gated_mlp", {"prefix": "m.", "hidden_size": 72, "intermediate_size": 200, "activation": "gelu_tanh"})
+    gelu = part_class("feed_forward", other)(other, rt)
+    gelu.bind(ws)
+    x = tensor((9, 72), rt, 8)
+    residual = torch.zeros((9, 72), dtype=torch.float32, device=x.device)
+    rt.ops.add_pending(residual, gelu.forward(x, residual))
+    g, u = f64(x) @ f64(ws["m.gate_proj.weight"]).T, f64(x) @ f64(ws["m.up_proj.weight"]).T
+    tanh_gelu = 0.5 * g * (1 + np.tanh(np.sqrt(2 / np.pi) * (g + 0.044715 * g**3)))
+    close(residual, (tanh_gelu * u) @ f64(ws["m.down_proj.weight"]).T, dtype, "feed-forward with the tanh form of GELU")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
