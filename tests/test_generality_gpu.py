@@ -1,7 +1,8 @@
 """A toy architecture, defined entirely in this test, is registered, built and stepped without a
 change to the framework's files: a mixer with fixed-size per-request state of its own, a feed-forward
 that routes each token to one of three experts, a position encoding of its own inside the stock
-attention mixer, and a run order that names one layer's weights twice and lets an entry read another
+attention mixer, a block arrangement of its own (mixer and feed-forward side by side behind one norm),
+and a run order that names one layer's weights twice and lets an entry read another
 entry's cache. Whole prompts, portions, single tokens and captured decode graphs must all agree with
 a plain implementation of the same toy, also defined here."""
 
@@ -23,7 +24,8 @@ ROT_DIM, POS_STEP = 8, 0.5  # the toy position encoding turns pair j of the firs
 @pytest.fixture(scope="module")
 def toy():
     from miniserve_amd.config import LayerSpec, ModelSpec, PartSpec, RunEntry, register_architecture, unregister_architecture
-    from miniserve_amd.parts import FeedForward, Mixer, PositionEncoding, Rotation, StateNeed, StateTensor, TensorSpec, register, unregister
+    from miniserve_amd.parts import (Block, FeedForward, Mixer, PositionEncoding, Rotation, StateNeed, StateTensor, TensorSpec, part_class,
+                                     register, unregister)
 
     @register("mixer", "toy_decay")
     class DecayMixer(Mixer):
@@ -121,6 +123,30 @@ def toy():
                 batch.memo[key] = torch.cat((torch.cos(ang), torch.sin(ang)), dim=1).contiguous()
             return Rotation(self.dim, batch.memo[key])
 
+    @register("block", "toy_side_by_side")
+    class SideBySide(Block):
+        """``h += mixer(norm(h)) + feed_forward(norm(h))``: one norm, both parts read its output."""
+
+        def __init__(self, spec, rt, mixer, feed_forward):
+            super().__init__(spec, rt, mixer, feed_forward)
+            n = spec["norm"]
+            self.norm = part_class("norm", n)(n, rt)
+
+        @classmethod
+        def tensors(cls, spec):
+            return dict(part_class("norm", spec["norm"]).tensors(spec["norm"]))
+
+        def bind(self, tensors):
+            self.norm.bind(tensors)
+
+        def forward(self, residual, batch, cache, state, pending=None):
+            x = self.norm.forward(residual, add=pending)
+            self.rt.ops.add_pending(residual, self.mixer.forward(x, batch, cache, state, residual))
+            return self.feed_forward.forward(x, residual)
+
+        def parameters_bytes(self):
+            return self.norm.parameters_bytes()
+
     @register_architecture("ToyForCausalLM")
     class ToyConfig:
         @classmethod
@@ -144,7 +170,7 @@ def toy():
                 "position": PartSpec("toy_slow_rotation", {"dim": ROT_DIM, "step": POS_STEP})})
             routed = PartSpec("toy_routed", {"width": H, "experts": EXPERTS, "inner": EXPERT_WIDTH, "router_scale": ROUTER_SCALE})
             layers = (
-                LayerSpec("l0.", block(), PartSpec("toy_decay", {"width": H, "decay": DECAY}), routed),
+                LayerSpec("l0.", PartSpec("toy_side_by_side", {"norm": norm("n1.weight")}), PartSpec("toy_decay", {"width": H, "decay": DECAY}), routed),
                 LayerSpec("l1.", block(), attn, ffn),
             )
             order = (RunEntry(0, 0), RunEntry(1, 1), RunEntry(1, 2), RunEntry(1, 1, writes_cache=False))
@@ -159,13 +185,14 @@ def toy():
     unregister("mixer", "toy_decay")
     unregister("feed_forward", "toy_routed")
     unregister("position", "toy_slow_rotation")
+    unregister("block", "toy_side_by_side")
 
 
 margins: list[float] = []  # smallest gap between the two best router logits of each sequence the plain toy ran
 
 
 def plain_toy(w, ids):
-    """The toy in float64: layer 0 (decay mixer, routed feed-forward), then layer 1's weights three
+    """The toy in float64: layer 0 (decay mixer and routed feed-forward side by side behind one norm), then layer 1's weights three
     times: with a cache of its own, with another cache of its own, and reading the keys and values of
     the first of these."""
     w = {k: v.double().cpu().numpy() for k, v in w.items()}
@@ -181,9 +208,9 @@ def plain_toy(w, ids):
     for t in range(T):
         s = DECAY * s + x[t]
         outs.append(s / (1 + (t + 1) / 8) + w["l0.toy.bias"])
-    h = h + np.stack(outs) @ w["l0.toy.weight"].T
-    # routed feed-forward: the expert with the largest router logit, weighted by its softmax weight
-    y = P.rms_norm(h, w["l0.n2.weight"], 1e-5)
+    mixed = np.stack(outs) @ w["l0.toy.weight"].T
+    # routed feed-forward on the same normalised input: the expert with the largest router logit, weighted by its softmax weight
+    y = x
     logits = (y @ w["l0.moe.router.weight"].T) * ROUTER_SCALE
     prob = np.exp(logits - logits.max(-1, keepdims=True))
     prob /= prob.sum(-1, keepdims=True)
@@ -193,7 +220,7 @@ def plain_toy(w, ids):
     w1 = w["l0.moe.w1.weight"].reshape(EXPERTS, EXPERT_WIDTH, H)
     w2 = w["l0.moe.w2.weight"].reshape(H, EXPERTS, EXPERT_WIDTH)
     out = np.stack([prob[t, e] * (w2[:, e, :] @ np.maximum(w1[e] @ y[t], 0.0)) for t, e in enumerate(choice)])
-    h = h + out
+    h = h + mixed + out
 
     ang = ((np.arange(T) * POS_STEP)[:, None] / np.arange(1, ROT_DIM // 2 + 1)[None, :]).astype(np.float32)
 
@@ -233,7 +260,18 @@ def test_toy_architecture_runs_through_the_engine(toy, dtype):
     cfg = config_from_dict({"architectures": ["ToyForCausalLM"]})
     spec = cfg.to_spec()
     rt = runtime(dtype)
-    weights = random_tensors(spec, 7, Init(0.08, (0.6, 1.4)), dtype=rt.dtype, device=rt.device)
+    # The comparison below means something only where rounding cannot change an expert choice: the first
+    # seed whose weights keep the router's two best logits apart at every position of the test's sequences.
+    rng = np.random.default_rng(3)
+    seqs = [rng.integers(0, VOCAB, n).tolist() for n in (37, 50, 9)]
+    for seed in range(7, 47):
+        weights = random_tensors(spec, seed, Init(0.08, (0.6, 1.4)), dtype=rt.dtype, device=rt.device)
+        margins.clear()
+        want = [plain_toy(weights, ids) for ids in seqs]
+        if min(margins) > (0.5 if dtype == "bfloat16" else 1e-3):
+            break
+    else:
+        pytest.fail(f"no seed keeps the router's choice clear of rounding (last margins {margins})")
     model = DecoderModel(spec, weights, rt)
     needs = model.cache_slots()
     assert [n.slot for n in needs] == [0, 1, 2] and needs[0].kv is None
@@ -243,12 +281,6 @@ def test_toy_architecture_runs_through_the_engine(toy, dtype):
 
     runner = ModelRunner(model, kv_pool_tokens=16 * 12, max_running=4, decode_graph=True)
     assert [g.slots for g in runner.layout.groups] == [(1, 2)] and [s.slot for s in runner.layout.states] == [0]
-    rng = np.random.default_rng(3)
-    seqs = [rng.integers(0, VOCAB, n).tolist() for n in (37, 50, 9)]
-    margins.clear()
-    want = [plain_toy(weights, ids) for ids in seqs]
-    # The comparison below means something only where rounding cannot change an expert choice.
-    assert min(margins) > (0.5 if dtype == "bfloat16" else 1e-3), f"router margins {margins}: pick another seed"
 
     def feed(rc, ids, at, n, wanted):
         return StepRow(rc, ids[at : at + n], wanted)
