@@ -102,7 +102,7 @@ __global__ __launch_bounds__(NT) void rmsnorm_kernel(float* __restrict__ x, cons
 
 // The same for few rows of a width that is a multiple of 4 and at most 8 NT, bfloat16 output: NT
 // threads per row, a thread owns up to two groups of 4 consecutive elements and moves them as vectors;
-// the partial sums of 8 splits are fetched at a time. Sums per element in ascending split order, as
+// the partial sums of up to 16 splits are fetched at a time. Sums per element in ascending split order, as
 // in the kernel above.
 // acc += parts of splits s0 .. s0 + B - 1 (those below `splits`), four floats each, in ascending order;
 // the B loads are issued before the first sum.
@@ -164,8 +164,10 @@ __global__ __launch_bounds__(NT) void rmsnorm_vec4_kernel(float* __restrict__ x,
           add_splits<2>(acc, p, 0, splits, split_stride);
         } else if (splits <= 4) {
           add_splits<4>(acc, p, 0, splits, split_stride);
-        } else {
-          for (int s0 = 0; s0 < splits; s0 += 8) add_splits<8>(acc, p, s0, splits, split_stride);
+        } else if (splits <= 8) {
+          add_splits<8>(acc, p, 0, splits, split_stride);
+        } else {  // the products of a decode step leave 12 to 16: one round trip, not two
+          for (int s0 = 0; s0 < splits; s0 += 16) add_splits<16>(acc, p, s0, splits, split_stride);
         }
         v.x += acc.x; v.y += acc.y; v.z += acc.z; v.w += acc.w;
         if (in_place) *reinterpret_cast<float4*>(src + i) = v;
