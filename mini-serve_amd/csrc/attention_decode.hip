@@ -621,23 +621,35 @@ __global__ __launch_bounds__(256) void attn_merge_project_kernel(const float* __
   }
 }
 
-// Heads per block so that the output projection's partial sums number at most 16.
-extern "C" int ms_attention_merge_project_splits(int Hq) {
+// Heads per block so that the output projection's partial sums number at most 16: 1, 2, 3 or 4 (a block's
+// slice of K, HB * D, is then a whole number of 64-element steps for both head sizes).
+static int merge_project_heads_per_block(int Hq) {
   const int hb = (Hq + 15) / 16;
-  return hb > MERGE_MAX_HB || Hq % hb ? -1 : Hq / hb;
+  return hb < 1 || hb > MERGE_MAX_HB || Hq % hb ? 0 : hb;
 }
 
-// P [ms_attention_merge_project_splits(Hq), rows, N] (float partial sums) from the split attention's
+// How many partial sums ms_attention_merge_project leaves for this shape, or -1 where it has no kernel and
+// the reduction kernel and the output projection must run apart. The one place that decides it: the launch
+// below asks the same function, so a caller that sizes its buffers by the answer is never refused afterwards.
+extern "C" int ms_attention_merge_project_splits(int rows, int Hq, int D, int splits, int N) {
+  const int hb = merge_project_heads_per_block(Hq);
+  if (hb == 0 || rows < 1 || rows > 16 || splits < 1 || splits > MERGE_MAX_SPLITS || (D != 64 && D != 128) || N <= 0 || N % 64)
+    return -1;
+  return Hq / hb;
+}
+
+// P [ms_attention_merge_project_splits(...), rows, N] (float partial sums) from the split attention's
 // partial results of `rows` <= 16 single-token rows (part_o, part_ml as the decode kernels leave them)
-// and the output projection's weight W [N, Hq * D]. MS_UNSUPPORTED where the two separate kernels must run.
+// and the output projection's weight W [N, Hq * D]. MS_UNSUPPORTED exactly where that function says -1.
+// The widest instance (D 128, 4 heads, 256 rows of W per block) holds its 256 registers of weights in the
+// vector registers and moves 68 values through the accumulation registers; nothing goes to scratch memory.
 extern "C" int ms_attention_merge_project(const float* part_o, const float* part_ml, const void* W, float* P, int rows,
                                           int Hq, int D, int splits, int N, hipStream_t st) {
   if (rows <= 0 || N <= 0) return MS_OK;
   if (part_o == nullptr || part_ml == nullptr || W == nullptr || P == nullptr || Hq <= 0 || splits < 1) return MS_BAD_ARG;
-  const int out_splits = ms_attention_merge_project_splits(Hq);
-  if (rows > 16 || splits > MERGE_MAX_SPLITS || (D != 64 && D != 128) || N % 64 || out_splits < 1) return MS_UNSUPPORTED;
+  const int out_splits = ms_attention_merge_project_splits(rows, Hq, D, splits, N);
+  if (out_splits < 1) return MS_UNSUPPORTED;
   const int hb = Hq / out_splits;
-  if ((hb * D) % 64 || (hb != 1 && hb != 2 && hb != 4)) return MS_UNSUPPORTED;
   // Rows of W per block: 64, or 256 where that still leaves a block for every CU.
   const int npw = (N % 256 == 0 && (long)out_splits * (N / 256) >= 256) ? 4 : 1;
   dim3 grid(out_splits, N / (64 * npw));
@@ -646,6 +658,7 @@ extern "C" int ms_attention_merge_project(const float* part_o, const float* part
 #define LAUNCH_HB(DD, NPW)                                                                                              \
   if (hb == 1) LAUNCH(DD, 1, NPW);                                                                                      \
   else if (hb == 2) LAUNCH(DD, 2, NPW);                                                                                 \
+  else if (hb == 3) LAUNCH(DD, 3, NPW);                                                                                 \
   else LAUNCH(DD, 4, NPW)
   if (D == 128 && npw == 4) { LAUNCH_HB(128, 4); }
   else if (D == 128) { LAUNCH_HB(128, 1); }

@@ -920,6 +920,18 @@ extern "C" int ms_gemm_bf16_tile_splits(int M, int N, int K) {
   return (slabs + per - 1) / per;  // no empty split
 }
 
+// Which tile ms_gemm_bf16 (gated == 0) or the tile form of ms_gemm_bf16_gated (gated != 0, N = 2 inter) runs a
+// product of these sizes with, as rows * 1000 + columns: 256256, 128064, 128128, 128160, 128192 or 64064 for the
+// kernel whose slabs go straight into LDS, 0 where K or the alignment sends the product to the kernel that
+// stages slabs through registers. For tests that must know which instance they have reached.
+extern "C" int ms_gemm_bf16_tile_shape(int M, int N, int K, int ldx, int splits, int gated) {
+  if (M <= 0 || N <= 0 || K <= 0 || splits < 1 || K % BK || ldx % 8) return 0;
+  const long big = (long)((M + 127) / 128) * ((N + 127) / 128) * splits;
+  if (big < 256) return 64064;
+  const int cols = pick_tile_cols(M, N, K, splits, gated != 0);
+  return cols == 256 ? 256256 : 128000 + cols;
+}
+
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T
 // splits > 1 (mode 1 only): C holds splits * M * N floats of partial sums, slice after slice.
 extern "C" int ms_gemm_bf16(const void* X, const void* W, void* C, int mode, int M, int N, int K, int ldx, int ldc,

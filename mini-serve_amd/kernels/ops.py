@@ -35,6 +35,7 @@ _SIGNATURES = {
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_tile_splits": [_c_int, _c_int, _c_int],
+    "ms_gemm_bf16_tile_shape": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_small_splits": [_c_int, _c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -46,7 +47,7 @@ _SIGNATURES = {
                                        _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
     "ms_attention_merge_project": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_attention_merge_project_splits": [_c_int],
+    "ms_attention_merge_project_splits": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "ms_attention_prefill_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int,
                                   _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_prefill_parts_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void,
@@ -387,6 +388,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
     return None if accumulate_into is not None else out
 
 
+def tile_shape(m: int, n: int, k: int, splits: int = 1, gated: bool = False) -> tuple[int, int] | None:
+    """``(rows, columns)`` of the tile that ``linear`` (or, with ``gated``, ``gated_linear`` with ``n = 2 I``)
+    runs a bfloat16 product of more than ``SMALL_M`` contiguous rows with; None where the shape takes the
+    kernel that stages its slabs through registers."""
+    code = library().ms_gemm_bf16_tile_shape(m, n, k, k, splits, int(gated))
+    return divmod(code, 1000) if code else None
+
+
 def add_pending(residual: torch.Tensor, pending: SplitSum | None) -> None:
     """``residual += pending`` for callers whose next kernel cannot take a pending sum itself."""
     if pending is None:
@@ -558,8 +567,8 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
             and t <= MERGE_PROJECT_MAX_ROWS):
         _dev(project, "project", BF16, 2)
         n = project.shape[0]
-        out_splits = lib.ms_attention_merge_project_splits(num_heads)
-        if project.shape[1] == num_heads * head_dim and n % 64 == 0 and out_splits >= 1:
+        out_splits = lib.ms_attention_merge_project_splits(t, num_heads, head_dim, splits, n)
+        if project.shape[1] == num_heads * head_dim and out_splits >= 1:
             merged = torch.empty((out_splits, t, n), dtype=F32, device=dev)
     out = None if merged is not None else torch.empty((t, num_heads * head_dim), dtype=BF16, device=dev)
     _check(lib.ms_attention_decode_fused_bf16(

@@ -134,7 +134,12 @@ def test_act_mul(ops, dtype, inter, act):
 # run the product and the activation as two kernels. All must agree.
 GATED = [(3000, 128, 4096), (1, 1024, 3072), (8, 1024, 3072), (16, 512, 64), (5, 2048, 160), (13, 4096, 48), (40, 1024, 3072), (64, 256, 64),
          (17, 1024, 3072), (32, 768, 160), (33, 512, 48), (64, 1024, 3072), (50, 2048, 64),
-         (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096)]
+         (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096),
+         (2048, 512, 12288), (4090, 512, 4080)]
+# The tile the activation's epilogue runs in, for the rows that are here for one (None: not asserted).
+GATED_TILES = {(3000, 128, 4096): (128, 128), (200, 1024, 3072): (64, 64), (2048, 1024, 3072): (128, 192),
+               (300, 192, 8192): (128, 64), (3000, 64, 4096): (128, 64),
+               (2048, 512, 12288): (256, 256), (4090, 512, 4080): (256, 256)}  # the last: ragged in both directions
 
 
 @pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
@@ -147,6 +152,8 @@ def test_gated_linear(ops, dtype, m, k, inter, act):
     want = activation(act, g) * u
     w = ops.interleave_gate_up(gate, up)
     assert w.shape == (2 * inter, k) and torch.equal(w[:16], gate[:16]) and torch.equal(w[16:32], up[:16])
+    if (m, k, inter) in GATED_TILES:
+        assert ops.tile_shape(m, 2 * inter, k, gated=True) == GATED_TILES[(m, k, inter)], "pick other sizes for this tile shape"
     got = ops.gated_linear(x, w, act, out_dtype=dtype, block=ops.GATE_BLOCK)
     assert got.shape == (m, inter) and got.dtype == dtype
     close(got, want, 1e-5 if dtype == F32 else 8e-3, f"gated {m}x{k}->{inter}")
@@ -189,22 +196,26 @@ def test_gemm_bf16(ops, m, n, k):
     close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
 
 
-@pytest.mark.parametrize("m,n,k", [(2000, 2100, 192), (4100, 1000, 64), (300, 14000, 320), (2048, 4096, 1024),
-                                   (4000, 1500, 192), (1990, 1000, 128), (2048, 6100, 128), (2048, 1000, 256),
-                                   (5000, 5000, 128), (4096, 4096, 64), (600, 33000, 192),
-                                   (1990, 5100, 512), (4100, 1000, 512), (4000, 4200, 1024), (600, 33000, 512),
-                                   (4090, 4090, 1024), (3000, 5000, 1024)])
-def test_gemm_bf16_large_tiles(ops, m, n, k):
-    """Shapes with at least 256 tiles of 128 x 128 and K a multiple of 64 take the kernel whose slabs go
-    straight into LDS: edge tiles in both directions (rows past the end are read from the last valid
-    row and never stored), one slab, an odd number of slabs. Which tile shape a product takes follows a
-    time model: with a short K the fixed part decides and most of the first row take 128 x 64 tiles, the
-    fourth and the last of the second row 128 x 128. (4000, 1500) and (1990, 1000) have many more rows
-    than columns and tile counts that divide by the XCD grid: each XCD then owns a rectangle of tiles,
-    with the matrix's edges in some of them. The third row: 128 x 160 tiles (32 columns of tiles, the last
-    one cut off, exactly 512 tiles; and 33 rows of 7 tiles), 128 x 192 tiles (many rows, and few rows of
-    a wide matrix). The last row: 256 x 256 tiles of eight waves (exactly one round of 256 with both edges
-    ragged, and 240 tiles)."""
+@pytest.mark.parametrize("m,n,k,tile", [
+    # a short K: the fixed part of the time decides, 128 x 64 tiles; edge tiles in both directions, one slab, an odd number of slabs
+    (2000, 2100, 192, (128, 64)), (4100, 1000, 64, (128, 64)), (300, 14000, 320, (128, 64)), (4000, 1500, 192, (128, 64)),
+    (2048, 6100, 128, (128, 64)), (5000, 5000, 128, (128, 64)), (4096, 4096, 64, (128, 64)),
+    (2048, 4096, 1024, (128, 128)), (600, 33000, 192, (128, 128)),
+    # fewer than 256 tiles of 128 x 128: 64 x 64 tiles of the same kernel
+    (1990, 1000, 128, (64, 64)), (2048, 1000, 256, (64, 64)),
+    # 128 x 160 (32 columns of tiles, the last one cut off, exactly 512 tiles; and 33 rows of 7 tiles)
+    (1990, 5100, 512, (128, 160)), (4100, 1000, 512, (128, 160)),
+    # 128 x 192 (many rows, and few rows of a wide matrix)
+    (4000, 4200, 1024, (128, 192)), (600, 33000, 512, (128, 192)),
+    # 256 x 256 tiles of eight waves (exactly one round of 256 with both edges ragged, and 240 tiles)
+    (4090, 4090, 1024, (256, 256)), (3000, 5000, 1024, (256, 256)),
+])
+def test_gemm_bf16_large_tiles(ops, m, n, k, tile):
+    """Every tile shape of the kernel whose slabs go straight into LDS (K a multiple of 64). Which shape a
+    product takes follows a fitted time model; the library says which it picks, and a row whose sizes no
+    longer reach the shape it is here for fails instead of testing another shape twice. Rows past the end
+    are read from the last valid row and never stored."""
+    assert ops.tile_shape(m, n, k) == tile, "this row no longer reaches the tile shape it was chosen for: pick other sizes"
     x, w = rand((m, k), BF16, 14), rand((n, k), BF16, 15)
     want = x.double() @ w.double().T
     close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"gemm bf16 {m}x{n}x{k} -> f32")
@@ -518,12 +529,99 @@ def test_decode_attention_bf16(ops, hq, hkv, d, lens_new, starts, window, boost)
     ],
 )
 @pytest.mark.parametrize("parts", ["host rule", "wherever possible"])
-def test_prefill_attention_bf16(ops, monkeypatch, hq, hkv, d, lens_new, starts, window, boost, parts):
+@pytest.mark.parametrize("tile_rows", [64, 128])
+def test_prefill_attention_bf16(ops, monkeypatch, hq, hkv, d, lens_new, starts, window, boost, parts, tile_rows):
     """``parts``: the keys of deep tiles are handed out in parts where the host's estimate says it pays, or
-    (second run) wherever a tile is deeper than the shortest part, so that small cases take that path too."""
+    (second run) wherever a tile is deeper than the shortest part, so that small cases take that path too.
+    ``tile_rows``: 64 query rows per block, as steps of this size run by themselves, or the 128-row blocks
+    (two wave groups that share a key tile and own 64 query rows each) that long steps take, forced here
+    by setting the number of blocks from which they run to zero."""
     if parts == "wherever possible":
         monkeypatch.setattr(ops, "PREFILL_PARTS_LAUNCH_US", -1e9)
+    if tile_rows == 128:
+        monkeypatch.setattr(ops, "PREFILL_BIG_BLOCKS", 0)
+    seen = spy_prefill_rows(ops, monkeypatch)
     attention_case(ops, BF16, hq, hkv, d, 16, lens_new, starts, window, seed=40, boost=boost)
+    assert seen == [tile_rows], seen
+
+
+def spy_prefill_rows(ops, monkeypatch) -> list:
+    """Records the query rows per block of every launch of the prefill attention."""
+    lib, seen = ops.library(), []
+    for name, at in (("ms_attention_prefill_bf16", 9), ("ms_attention_prefill_parts_bf16", 11)):
+        real = getattr(lib, name)
+
+        def wrapped(*args, _real=real, _at=at):
+            seen.append(args[_at])
+            return _real(*args)
+
+        monkeypatch.setattr(lib, name, wrapped)
+    return seen
+
+
+@pytest.mark.parametrize(
+    "hq,hkv,d,lens_new,starts,boost",
+    [
+        (64, 8, 128, [1300], [0], (0, 70)),            # a step long enough for 128-row blocks by its own size
+        (16, 8, 128, [5200, 1], [40, 3000], (0, 11)),  # two heads per group: 64 tokens per block, beside a decode row
+    ],
+)
+def test_prefill_attention_128_row_blocks_by_size(ops, monkeypatch, hq, hkv, d, lens_new, starts, boost):
+    """Steps that reach the 128-row blocks under the host's own rule, nothing forced. Only the last 70
+    tokens of the long row and the far key are checked against the slow reference (the whole step would
+    take it minutes); the rest against the 64-row blocks, which the cases above pin."""
+    seen = spy_prefill_rows(ops, monkeypatch)
+    got = attention_tail_case(ops, hq, hkv, d, lens_new, starts, boost, check_last=70)
+    assert seen == [128], seen
+    monkeypatch.setattr(ops, "PREFILL_BIG_BLOCKS", 1 << 30)
+    small = attention_tail_case(ops, hq, hkv, d, lens_new, starts, boost, check_last=0)
+    assert seen == [128, 64], seen
+    close(got, small, 8e-3, "128-row blocks against 64-row blocks, every token")
+
+
+def attention_tail_case(ops, hq, hkv, d, lens_new, starts, boost, check_last):
+    """As ``attention_case`` in bfloat16 with 16-token pages, but only the last ``check_last`` tokens of row 0 are
+    compared with the float64 reference. Returns the kernel's output."""
+    page, seed = 16, 50
+    g = torch.Generator().manual_seed(seed)
+    totals = [s + n for s, n in zip(starts, lens_new)]
+    blocks = [-(-tt // page) for tt in totals]
+    pages = sum(blocks) + 3
+    order = torch.randperm(pages, generator=g).tolist()
+    table = torch.full((len(lens_new), max(blocks)), -1, dtype=torch.int32)
+    kc, vc = rand((pages, hkv, page, d), BF16, seed + 1), rand((pages, hkv, d, page), BF16, seed + 2)
+    at = 0
+    for i, nb in enumerate(blocks):
+        table[i, :nb] = torch.tensor(order[at : at + nb], dtype=torch.int32)
+        at += nb
+    t = sum(lens_new)
+    q = rand((t, (hq + 2 * hkv) * d), BF16, seed + 3)
+    row, where = boost
+    last = sum(lens_new[: row + 1]) - 1
+    key = kc[table[row, where // page], :, where % page]
+    qv = q[last].view(hq + 2 * hkv, d)
+    for h in range(hq):
+        qv[h] = (key[h // (hq // hkv)].float() * 3.0).to(BF16)
+    scale = d**-0.5
+    got = ops.paged_attention(q, kc, vc, table.to(DEV), make_batch(lens_new, starts), hq, hkv, d, scale, 0)
+    if check_last:
+        n0, total = lens_new[0], totals[0]
+        idx = table[0].long().to(DEV)
+        keys = kc[idx].permute(0, 2, 1, 3).reshape(-1, hkv, d)[:total].double()  # [len, hkv, d]
+        vals = vc[idx].permute(0, 3, 1, 2).reshape(-1, hkv, d)[:total].double()
+        qd = q.double().view(t, hq + 2 * hkv, d)[:, :hq]
+        want = torch.empty((check_last, hq, d), dtype=torch.float64, device=DEV)
+        for j in range(check_last):
+            tok = n0 - check_last + j
+            p = starts[0] + tok
+            for h in range(hq):
+                kh = h // (hq // hkv)
+                wgt = torch.softmax((keys[: p + 1, kh] @ qd[tok, h]) * scale, 0)
+                if tok == n0 - 1:
+                    assert float(wgt[where]) > 0.9, "the boosted key was meant to dominate"
+                want[j, h] = wgt @ vals[: p + 1, kh]
+        close(got.view(t, hq, d)[n0 - check_last : n0], want, 8e-3, f"attention {hq}/{hkv}/{d}, the row's last tokens")
+    return got
 
 
 def test_prefill_attention_parts_are_taken(ops, monkeypatch):
@@ -548,6 +646,10 @@ def test_prefill_attention_parts_are_taken(ops, monkeypatch):
         (6, 6, 64, [300, 40, 41, 1200], 100, True, True),              # one head per group, a window
         (16, 8, 128, [500, 31, 2047], 33, True, True),
         (4, 2, 128, list(range(0, 6400, 100)), 0, True, True),         # a full batch: one split
+        (48, 8, 128, [700, 3000], 0, True, True),                      # three heads per block of the merged projection
+        (48, 4, 64, [513, 77, 5], 0, True, True),                      # the same at head size 64, twelve heads per group
+        (36, 12, 64, [900, 40], 0, False, True),
+        (40, 8, 128, [400, 1300], 0, True, True),                      # 40 heads: no whole number of blocks of three
     ],
 )
 def test_decode_attention_fused(ops, hq, hkv, d, starts, window, norm, rot):
@@ -610,7 +712,7 @@ def test_decode_attention_fused(ops, hq, hkv, d, starts, window, norm, rot):
         k4, v4 = kc.clone(), vc.clone()
         got = ops.decode_attention_fused(ops.SplitSum(parts), qw, kw, eps, rope, True, k4, v4, table, batch, hq, hkv, d, scale,
                                          window, project=wo)
-        if b <= 16 and 1 < splits <= 64:
+        if b <= 16 and 1 < splits <= 64 and hq != 40:
             assert isinstance(got, ops.SplitSum) and got.shape == (b, n) and got.splits <= 16
             close(got.parts.double().sum(0), want.double() @ wo.double().T, 1e-2, f"reduction of the splits and projection in one, {n}")
             assert torch.equal(flat(k4, False)[sl], flat(k2, False)[sl]) and torch.equal(flat(v4, True)[sl], flat(v2, True)[sl])

@@ -111,3 +111,42 @@ def test_layer_sizes_of_the_benchmark_shapes(shape):
     mixed, single = run(m, ids, [200, 60, 40], last, beside=(ids2, 1))
     check_logits(mixed.numpy(), want, "bfloat16", f"{name} shape bfloat16 mixed")
     check_logits(single.numpy(), want2, "bfloat16", f"{name} shape bfloat16, a single token beside a portion")
+
+
+def test_a_2048_token_step_of_the_32B_layer(shape, monkeypatch):
+    """One step of 2,048 prompt tokens at the 32B layer sizes, bfloat16: eight query heads per KV head make
+    16-token attention blocks, 1,024 of them, so this step (and every step of that shape's benchmark) runs
+    the prefill attention's 128-row blocks and the matrix products' largest tiles. The last 40 positions'
+    logits against the plain implementation."""
+    name, cfg, spec, tensors, w = shape
+    if name != "32B":
+        pytest.skip("only the 32B shape's group of eight heads reaches the 128-row blocks at 2,048 tokens")
+    from miniserve_amd.kernels import ops
+
+    lib, seen = ops.library(), []
+    for fn, at in (("ms_attention_prefill_bf16", 9), ("ms_attention_prefill_parts_bf16", 11)):
+        real = getattr(lib, fn)
+        monkeypatch.setattr(lib, fn, lambda *a, _real=real, _at=at: (seen.append(a[_at]), _real(*a))[1])
+    rng = np.random.default_rng(2)
+    T, last = 2048, 40
+    ids = rng.integers(0, 150000, T).tolist()
+    c = P.read_config(cfg)
+    h = P.hidden_states(cfg, w, ids)[T - last :]
+    want = P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["lm_head.weight"].T
+    m = model(spec, tensors, "bfloat16")
+    from miniserve_amd.engine.batch import StepRow
+    from miniserve_amd.engine.runner import ModelRunner
+
+    runner = ModelRunner(m, kv_pool_tokens=4096, max_running=2)
+    rc = runner.acquire()
+    got = runner.step([StepRow(rc, ids, list(range(T - last, T)))]).float().cpu().numpy()
+    assert seen and set(seen) == {128}, seen
+    check_logits(got, want, "bfloat16", "32B shape bfloat16, 2,048 tokens in one step")
+    # and the next portion behind it, beside nothing: 600 more tokens whose blocks (38 x 8) are few again
+    more = rng.integers(0, 150000, 600).tolist()
+    h = P.hidden_states(cfg, w, ids + more)[-last:]
+    want = P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["lm_head.weight"].T
+    got = runner.step([StepRow(rc, more, list(range(600 - last, 600)))]).float().cpu().numpy()
+    assert seen[-1] == 64, seen
+    check_logits(got, want, "bfloat16", "32B shape bfloat16, 600 tokens behind 2,048")
+    runner.release(rc)
