@@ -6,13 +6,15 @@ bfloat16, batch 8 at a context of 4,096 tokens per request, 16-token pages.
 A "step" is one decode step of the engine (schedule, one pass of the model over the batch's last
 tokens, sampling on the device, one read-back of the tokens, which the engine waits for one step
 after the launch). Requests are prefilled through the same step function in portions of 2,048 tokens;
-the timed steps are the last K before every request reaches the context length. Before them run at
-least W untimed decode steps and at least ``--warmup-seconds`` of them (the number is fixed before the
-prompts are made, from a floor on the step time, so that the timed steps end at the context length;
-what the GPU's clock did meanwhile is in ``sidecar``).
+the timed steps are the last K before every request reaches the context length. Before them run W
+untimed decode steps, and then the last of them is run again and again on the same inputs (the same
+kernels at the same context; nothing advances, so the timed steps still end at the context length)
+for at least ``--warmup-seconds`` and until the GPU's shader clock has stopped moving, at most
+``--warmup-most-seconds``; what the clock, the power and the temperatures did meanwhile is in ``sidecar``.
 
 One JSON line is printed. ``value`` = decoded tokens per second of the headline point. Beside it:
-``prefill`` (one 2,048-token prompt in one step; median of five), ``roofline`` (the decode step's bytes,
+``prefill`` (one 2,048-token prompt in one step; median of five; its flops are what the model's parts say
+of themselves), ``roofline`` (the decode step's bytes,
 every weight once plus the live requests' cache, over its time, against the published 8 TB/s),
 ``points`` (decode at batch 1 and 64 of the same shape; unless ``--no-extra``, decode at batch 8 behind
 32,768 tokens and a prompt of 8,192 tokens in one step, the Qwen3-8B shape's decode at batch 1 / 8 / 64, its
@@ -41,7 +43,6 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
-STEP_TIME_FLOOR_S = 1.0e-3  # no decode step of these shapes is faster: sizes the warm-up by time
 
 
 def say(msg):
@@ -53,7 +54,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--warmup-seconds", type=float, default=0.3, help="decode for at least this long before the timed steps")
+    ap.add_argument("--warmup-seconds", type=float, default=0.3,
+                    help="after the warm-up steps, repeat the last of them for at least this long and until the clock is steady")
+    ap.add_argument("--warmup-most-seconds", type=float, default=3.0, help="give up waiting for a steady clock after this long")
     ap.add_argument("--preset", default="0.6B")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the preset has (reported in config)")
     ap.add_argument("--batch", type=int, default=8)
@@ -79,7 +82,7 @@ def main() -> int:
     from miniserve_amd.engine.request import RequestState, SamplingParams
     from miniserve_amd.engine.runner import ModelRunner
     from miniserve_amd.loading import random_model
-    from miniserve_amd.measurement import GpuSampler, measured_region, sidecar
+    from miniserve_amd.measurement import GpuMonitor, measured_region, sidecar
     from miniserve_amd.measurement.offline import run_to_completion
 
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
@@ -96,11 +99,11 @@ def main() -> int:
         say(f"building the {name} shape ({cfg['num_hidden_layers']} of {full} layers, {args.dtype})")
         return cfg, full, random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
 
-    def decode_run(model, cfg, batch, steps, warmup, sampler=None, describe=False, context=None):
+    def decode_run(model, cfg, batch, steps, warmup, describe=False, context=None):
         """Decode ``steps`` timed tokens for ``batch`` requests ending at the context length, after the
         warm-up; returns a dict with the rate, the step time and the step's share of the roofline."""
         context = context or args.context
-        warm_steps = max(warmup, math.ceil(args.warmup_seconds / STEP_TIME_FLOOR_S))
+        warm_steps = max(warmup, 1)
         total = warm_steps + steps
         # Decoding requests keep decoding while later ones are still prefilled (a step per 2,048 prompt
         # tokens of each): prompts are shortened by that much, so that the longest sequence ends at the
@@ -125,10 +128,17 @@ def main() -> int:
         for _ in range(warm_steps):
             eng.step()
         torch.cuda.synchronize()
+
+        def hold():  # the latest step again, a few times: the device stays at the step's load, the context stays put
+            for _ in range(8):
+                eng.runner.repeat_last_step()
+            torch.cuda.synchronize()
+
+        held = monitor.warm_until_steady(hold, args.warmup_seconds, max(args.warmup_seconds, args.warmup_most_seconds))
         warm_s = time.perf_counter() - w0
-        settled = sampler.settled() if sampler is not None else None
+        monitor.interval_s = 0.1  # fewer readings while the host is being timed
         ctx0 = sum(r.seq_len for r in reqs) / batch
-        t_mark = sampler.sample_now() if sampler is not None else time.monotonic()
+        t_mark = monitor.read_now()
         with measured_region(f"decode b{batch}"):
             t0 = time.perf_counter()
             for _ in range(steps):
@@ -140,7 +150,8 @@ def main() -> int:
         step_bytes = model.decode_read_bytes() + batch * mean_ctx * eng.runner.pool.bytes_per_token()
         out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "mean_ctx": mean_ctx,
                "achieved_gbs": step_bytes / (dt / steps) / 1e9, "warmup_steps": warm_steps, "warmup_s": round(warm_s, 3),
-               "clock_settled": settled, "since": t_mark, "until": sampler.sample_now() if sampler is not None else time.monotonic()}
+               "held": held, "since": t_mark, "until": monitor.read_now()}
+        monitor.interval_s = 0.02
         if describe:
             out["sidecar"] = sidecar(eng)
         for r in reqs:
@@ -167,12 +178,9 @@ def main() -> int:
                 times.append(time.perf_counter() - t0)
             runner.release(rc)
         pre = statistics.median(times[1:])
-        L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
-        Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-        linear = 2 * T * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I) + 2 * H * vocab
-        attn = 2 * T * (T + 2 * C) * D * Hq * L  # causal: QK^T and PV over half the square each, and over the cached keys
+        # every matrix product of the T tokens, both attention products over each (query, visible key) pair, the head once
         out = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
-               "frac": round((linear + attn) / pre / PEAK_FLOPS[dt_name], 4)}
+               "frac": round(model.step_flops([(T, C)]) / pre / PEAK_FLOPS[dt_name], 4)}
         if C:
             out["cached"] = C
         del runner
@@ -181,7 +189,7 @@ def main() -> int:
     def continuous_run(model, cfg, requests=64, prompt_len=2048, new_tokens=512, budget=512):
         """The reference's offline workload for its largest model: all requests at once, prompts cut into
         portions under a step budget and mixed with decoding requests. Decode-only and mixed steps are
-        timed apart; a mixed step's flops are its tokens' linear products (attention aside)."""
+        timed apart; a mixed step's flops are what the model's parts say of its rows (attention included)."""
         eng = Engine(model, max_running=requests, kv_pool_tokens=requests * (prompt_len + new_tokens + 32),
                      chunked_prefill_size=budget, decode_graph=not args.no_graph)
         for p in prompts(cfg["vocab_size"], requests, prompt_len):
@@ -192,9 +200,6 @@ def main() -> int:
         assert eng.runner.cache.idle
         weights = model.decode_read_bytes()
         per_tok = eng.runner.pool.bytes_per_token()
-        L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
-        Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-        flops_per_token = 2 * L * (H * (Hq + 2 * Hkv) * D + Hq * D * H + 3 * H * I)
         out = {"tok_s": requests * new_tokens / ran["seconds"], "seconds": ran["seconds"], "preemptions": eng.scheduler.num_preemptions}
         d, m = ran["decode"], ran["mixed"]
         if d["steps"]:
@@ -205,7 +210,7 @@ def main() -> int:
         if m["steps"]:
             out["mixed_step_ms"] = m["median_ms"]
             out["mixed_tokens"] = m["mean_tokens"]
-            out["mixed_frac_flops"] = flops_per_token * m["mean_tokens"] / (m["median_ms"] * 1e-3) / PEAK_FLOPS[dt_name]
+            out["mixed_frac_flops"] = m["mean_flops"] / (m["median_ms"] * 1e-3) / PEAK_FLOPS[dt_name]
             out["mixed_frac_hbm"] = weights / (m["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
         del eng
         return out
@@ -213,15 +218,15 @@ def main() -> int:
     cfg, full_layers, model = make(args.preset, args.layers)
     vocab = cfg["vocab_size"]
     side = {}
+    monitor = GpuMonitor().start()  # readings every 20 ms from here to the end of the run
     if args.prefill_only:
         head = {"tok_s": 0.0, "ms_per_step": 0.0, "achieved_gbs": 0.0, "mean_ctx": 0.0, "warmup_steps": 0}
     else:
-        with GpuSampler() as gpu:
-            head = decode_run(model, cfg, args.batch, args.steps, args.warmup, sampler=gpu, describe=True)
-            side = head.pop("sidecar")
-            side["warmup"] = {"steps": head["warmup_steps"], "seconds": head["warmup_s"], "clock_settled": head["clock_settled"]}
-            side["gpu_during_timed_steps"] = gpu.summary(head["since"], head["until"])
-            side["gpu_during_run"] = gpu.summary()
+        head = decode_run(model, cfg, args.batch, args.steps, args.warmup, describe=True)
+        side = head.pop("sidecar")
+        side["warmup"] = {"steps": head["warmup_steps"], "seconds": head["warmup_s"], "repeats_of_the_last_step": 8 * head["held"]["calls"],
+                          "held_seconds": head["held"]["seconds"], "clock_steady": head["held"]["steady"]}
+        side["gpu_during_timed_steps"] = monitor.window(head["since"], head["until"])
     achieved = head["achieved_gbs"]
 
     out = {
@@ -271,14 +276,16 @@ def main() -> int:
         n = 1 << 30
         buf = torch.empty((n,), dtype=torch.uint8, device="cuda:0").random_(0, 256)
         read = n / median_ms(lambda: ops.measure_read(buf)) / 1e6
-        del buf
+        dst = torch.empty_like(buf)
+        copy = 2 * n / median_ms(lambda: ops.measure_copy(buf, dst)) / 1e6  # bytes read plus bytes written
+        del buf, dst
         rates = {}
         for n in (4096, 8192):
             x = torch.randn((n, n), device="cuda:0").to(torch.bfloat16)
             w = torch.randn((n, n), device="cuda:0").to(torch.bfloat16)
             rates[n] = 2 * n**3 / median_ms(lambda: ops.linear(x, w, out_dtype=torch.bfloat16)) / 1e9
             del x, w
-        out["measured_peaks"] = {"read_GBps": round(read, 1), "gemm_bf16_4096_TFLOPs": round(rates[4096], 1),
+        out["measured_peaks"] = {"read_GBps": round(read, 1), "copy_GBps": round(copy, 1), "gemm_bf16_4096_TFLOPs": round(rates[4096], 1),
                                  "gemm_bf16_8192_TFLOPs": round(rates[8192], 1),
                                  "decode_frac_of_read": round(achieved / read, 4)}
 
@@ -319,7 +326,10 @@ def main() -> int:
         gc.collect()
         torch.cuda.empty_cache()
 
+    monitor.stop()
     if side:
+        side["gpu_during_run"] = monitor.window()
+        side["conditions"] = monitor.conditions()
         out["sidecar"] = side
     print(json.dumps(out))
     return 0

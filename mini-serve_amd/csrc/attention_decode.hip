@@ -469,16 +469,17 @@ extern "C" int ms_attention_decode_bf16(const void* q, int q_stride, const void*
 // The same over the qkv projection's partial sums `parts` [qkv_splits, tokens, (Hq + 2 Hkv) D] (floats,
 // qkv_split_stride apart) of a step whose rows bring one token each: per-head RMSNorm of q and k with
 // bfloat16 weights [D] (both nullptr: none), rotation over the whole head by the table `rope`
-// [tokens, D] (nullptr: none), and, with store != 0, the new token's key and value written to its place
+// [tokens, D] (nullptr: none) in pairs (j, j + D/2) (rope_pairing must be MS_ROPE_HALVES: the kernel's lanes
+// hold the halves of a head side by side; any other pairing is MS_UNSUPPORTED), and, with store != 0, the new token's key and value written to its place
 // in the cache (its page is taken from the block table at pos).
 extern "C" int ms_attention_decode_fused_bf16(const float* parts, int qkv_splits, long long qkv_split_stride,
                                               const void* q_weight, const void* k_weight, float eps, const float* rope,
-                                              int store, void* kc, void* vc, const int* block_table, int table_width,
+                                              int rope_pairing, int store, void* kc, void* vc, const int* block_table, int table_width,
                                               const int* tokens, const int* token_row, const int* pos, void* out,
                                               float* part_o, float* part_ml, int rows, int splits, int Hq, int Hkv, int D,
                                               int page_size, float scale, int window, int reduce, hipStream_t st) {
   if (rows <= 0) return MS_OK;
-  if (page_size != PAGE || (D != 64 && D != 128)) return MS_UNSUPPORTED;
+  if (page_size != PAGE || (D != 64 && D != 128) || (rope != nullptr && rope_pairing != MS_ROPE_HALVES)) return MS_UNSUPPORTED;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || splits < 1 || splits > 65535 || window < 0 || table_width <= 0 ||
       (splits > 1 && (!part_o || !part_ml)) || (splits > 1 && reduce && out == nullptr) || (splits == 1 && out == nullptr) ||
       parts == nullptr || qkv_splits < 1 || qkv_split_stride % 4 ||

@@ -76,6 +76,10 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ p, int spl
   return acc;
 }
 
+// Which elements of a head make pair j of a rotary position encoding: (j, j + rot/2) or (2j, 2j + 1).
+#define MS_ROPE_HALVES 0
+#define MS_ROPE_ADJACENT 1
+
 // Activations of the gated feed-forward, by the number the host passes: out = act(gate) * up, in float32.
 #define MS_ACT_SILU 0
 #define MS_ACT_GELU_TANH 1

@@ -339,7 +339,8 @@ extern "C" int ms_rope_table(const int* pos, const float* inv_freq, float* out, 
 // Head slots [0, Hq) are query heads, [Hq, Hq+Hkv) key heads, [Hq+Hkv, Hq+2Hkv) value heads of the
 // token's row in qkv [tokens, (Hq + 2 Hkv) * D].
 //   q, k: optional RMSNorm over the head (weight [D]), then rotation of the first `rot` elements in
-//         pairs (j, j + rot/2) by the angle whose cosine and sine are rope[t][j] and rope[t][rot/2 + j];
+//         pairs by the angle whose cosine and sine are rope[t][j] and rope[t][rot/2 + j] for pair j: the
+//         elements (j, j + rot/2) (MS_ROPE_HALVES) or (2j, 2j + 1) (MS_ROPE_ADJACENT);
 //   q goes to q_out; k and v go to the cache page of the token's slot
 //   (slot = page * page_size + offset; keys [pages, Hkv, page_size, D], values transposed within
 //   the page, [pages, Hkv, D, page_size]).
@@ -352,8 +353,8 @@ template <typename T, typename TW>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const T* qkv, const float* __restrict__ parts, int splits, size_t split_stride, T* q_out, int q_out_stride,
     const int* __restrict__ slots, const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
-    const float* __restrict__ rope, int rot, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D, int page_size,
-    int heads) {
+    const float* __restrict__ rope, int rot, int pairing, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D,
+    int page_size, int heads) {
   __shared__ float buf[4][MAX_HEAD_DIM];
   const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int hs = blockIdx.y * 4 + wave;  // this wave's head slot
@@ -414,8 +415,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
         for (int i = 0; i < PER; ++i) {
           const int e = lane + i * WAVE;
           if (e < rot) {
-            const int j = e < half ? e : e - half;
-            x[i] = e < half ? x[i] * cs[j] - buf[wave][e + half] * sn[j] : x[i] * cs[j] + buf[wave][e - half] * sn[j];
+            // first of its pair: x cos - partner sin; second: x cos + partner sin
+            const bool first = pairing == MS_ROPE_ADJACENT ? (e & 1) == 0 : e < half;
+            const int j = pairing == MS_ROPE_ADJACENT ? e / 2 : (e < half ? e : e - half);
+            const int partner = pairing == MS_ROPE_ADJACENT ? (e ^ 1) : (e < half ? e + half : e - half);
+            x[i] = first ? x[i] * cs[j] - buf[wave][partner] * sn[j] : x[i] * cs[j] + buf[wave][partner] * sn[j];
           }
         }
         __builtin_amdgcn_wave_barrier();
@@ -606,23 +610,25 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_tile_kernel(
 
 // Source: qkv [tokens, (Hq + 2 Hkv) D], or (parts != nullptr) float partial sums [splits, tokens, (Hq + 2 Hkv) D] of it.
 // Queries go to q_out [tokens, q_out_stride >= Hq D] (which may be qkv itself: in place). rope is the
-// table of ms_rope_table for these tokens with half = rot / 2 (nullptr when rot == 0).
+// table of ms_rope_table for these tokens with half = rot / 2 (nullptr when rot == 0), pairing an MS_ROPE_*
+// number (MS_UNSUPPORTED for any other).
 extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int splits, long long split_stride, void* q_out,
                                      int q_out_stride, int is_bf16, const int* slots, const void* qw, const void* kw,
-                                     int w_is_bf16, float eps, const float* rope, int rot, void* kc, void* vc, int tokens,
-                                     int Hq, int Hkv, int D, int page_size, hipStream_t st) {
+                                     int w_is_bf16, float eps, const float* rope, int rot, int pairing, void* kc, void* vc,
+                                     int tokens, int Hq, int Hkv, int D, int page_size, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if ((qkv == nullptr) == (parts == nullptr) || (parts != nullptr && splits < 1) || q_out == nullptr || q_out_stride < Hq * D)
     return MS_BAD_ARG;
   if (D <= 0 || D > MAX_HEAD_DIM || rot < 0 || rot > D || (rot & 1) || Hq <= 0 || Hkv <= 0 || page_size <= 0) return MS_BAD_ARG;
   if ((qw == nullptr) != (kw == nullptr)) return MS_BAD_ARG;
   if ((rot > 0) != (rope != nullptr)) return MS_BAD_ARG;
+  if (rot > 0 && pairing != MS_ROPE_HALVES && pairing != MS_ROPE_ADJACENT) return MS_UNSUPPORTED;
   const int heads = slots ? Hq + 2 * Hkv : Hq;
   if ((heads + 3) / 4 > 65535 || heads > 65535) return MS_BAD_ARG;
   // The tile kernel moves 8 elements at a time: every row it touches must start on such a boundary.
   // Which kernel runs depends on the head's shape alone, never on the number of tokens: a token's
   // result is the same bit for bit in whatever step it comes.
-  const bool tiled = (D == 64 || D == 128) && (rot == 0 || rot == D) && q_out_stride % 8 == 0 &&
+  const bool tiled = (D == 64 || D == 128) && (rot == 0 || (rot == D && pairing == MS_ROPE_HALVES)) && q_out_stride % 8 == 0 &&
                      (parts == nullptr || split_stride % 4 == 0);
   if (tiled) {
     const int tok_per_block = 256 / (D / 8);
@@ -651,7 +657,7 @@ extern "C" int ms_qk_norm_rope_store(const void* qkv, const float* parts, int sp
 #define LAUNCH(T, TW)                                                                                                   \
   qk_norm_rope_store_kernel<T, TW><<<dim3(tokens, (heads + 3) / 4), 256, 0, st>>>(                                      \
       (const T*)qkv, parts, splits, (size_t)split_stride, (T*)q_out, q_out_stride, slots, (const TW*)qw, (const TW*)kw, \
-      eps, rope, rot, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
+      eps, rope, rot, pairing, (T*)kc, (T*)vc, Hq, Hkv, D, page_size, heads)
   if (is_bf16 && w_is_bf16) LAUNCH(bf16, bf16);
   else if (is_bf16) LAUNCH(bf16, float);
   else if (w_is_bf16) LAUNCH(float, bf16);

@@ -5,7 +5,6 @@ which graphs exist), not on the command line. Same idea and keys as the referenc
 
 from __future__ import annotations
 
-import subprocess
 from pathlib import Path
 
 
@@ -42,28 +41,41 @@ def engine_description(engine) -> dict:
     return out
 
 
+def _checkout_commit(root: Path) -> str | None:
+    """The commit a checkout stands at, read from its ``.git`` folder (no git program needed); None
+    where the tree is no checkout."""
+    try:
+        head = (root / ".git" / "HEAD").read_text().strip()
+        if not head.startswith("ref:"):
+            return head or None
+        ref = head.split(None, 1)[1]
+        loose = root / ".git" / ref
+        if loose.is_file():
+            return loose.read_text().strip() or None
+        for line in (root / ".git" / "packed-refs").read_text().splitlines():
+            if line.endswith(" " + ref):
+                return line.split()[0]
+    except OSError:
+        pass
+    return None
+
+
 def runtime_description() -> dict:
-    """The software and the device underneath, for the same record."""
+    """What the engine stands on: the device as the HIP runtime describes it, the library versions, and
+    which build of the kernel sources is loaded (its file name carries the digest of the sources, so it
+    identifies the code even where the tree is a bare copy without history)."""
     import torch
 
-    def git(*args: str):
-        try:
-            root = Path(__file__).resolve().parents[2]
-            return subprocess.run(["git", "-C", str(root), *args], capture_output=True, text=True, check=True, timeout=10).stdout.strip()
-        except Exception:  # noqa: BLE001  (a checkout is not always there)
-            return None
-
-    props = torch.cuda.get_device_properties(0) if torch.cuda.is_available() else None
     from ..kernels import build
 
-    return dict(
-        torch=torch.__version__,
-        hip=getattr(torch.version, "hip", None),
-        gpu=None if props is None else props.name,
-        gpu_arch=None if props is None else getattr(props, "gcnArchName", None),
-        gpu_memory_bytes=None if props is None else props.total_memory,
-        compute_units=None if props is None else props.multi_processor_count,
-        kernel_library=build.kernel_library_name(),
-        git_commit=git("rev-parse", "HEAD"),
-        git_dirty=bool(git("status", "--porcelain", "--untracked-files=no")),
-    )
+    record = {"torch": torch.__version__, "hip": getattr(torch.version, "hip", None)}
+    device = {"gpu": None, "gpu_arch": None, "gpu_memory_bytes": None, "compute_units": None, "l2_cache_bytes": None}
+    if torch.cuda.is_available():
+        p = torch.cuda.get_device_properties(0)
+        device = {"gpu": p.name, "gpu_arch": getattr(p, "gcnArchName", None), "gpu_memory_bytes": p.total_memory,
+                  "compute_units": p.multi_processor_count, "l2_cache_bytes": getattr(p, "L2_cache_size", None)}
+    record.update(device)
+    record["kernel_library"] = build.kernel_library_name()
+    record["block_core_library"] = build.core_library_name()
+    record["commit"] = _checkout_commit(Path(__file__).resolve().parents[2])
+    return record

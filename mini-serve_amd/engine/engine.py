@@ -87,6 +87,7 @@ class Engine:
                 kv_mem_fraction=kv_mem_fraction,
                 max_running=max_running,
                 max_step_tokens=chunked_prefill_size or max_prefill_tokens,
+                request_step_tokens=chunked_prefill_size or None,  # whole prompts run in one step, however long
                 allocator_class=allocator_class(block_backend),
                 decode_graph=decode_graph,
                 decode_graph_max_bs=decode_graph_max_bs,

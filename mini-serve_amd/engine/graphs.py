@@ -45,6 +45,7 @@ class DecodeGraphs:
         self.max_bs = max_bs
         self.captured: dict = {}
         self.pool = None
+        self.latest = None  # the captured graph the latest ``run`` replayed
         self.num_groups = len(runner.layout.groups)
 
     def usable(self, rows) -> bool:
@@ -175,4 +176,5 @@ class DecodeGraphs:
             o, n = c.seg["feed"]
             self.runner.model.rt.ops.feed_tokens(c.batch.token_ids, None, c.dev[o : o + n], feed_from)
         c.graph.replay()
+        self.latest = c
         return c.logits[:B]

@@ -30,7 +30,7 @@ _SIGNATURES = {
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
     "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
-                              _c_int, _c_float, _c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_int, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
     "ms_gemm_f32": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -43,7 +43,7 @@ _SIGNATURES = {
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
-    "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_void,
+    "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void,
                                        _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
     "ms_attention_merge_project": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -422,10 +422,23 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
     return out
 
 
+# Which elements of a head make pair j of a rotation, and the numbers the kernels know the pairings by (MS_ROPE_* in
+# csrc/common.h): "halves" (j, j + dim/2), "adjacent" (2j, 2j + 1).
+ROTATION_PAIRINGS = {"halves": 0, "adjacent": 1}
+
+
+def _pairing(name: str) -> int:
+    try:
+        return ROTATION_PAIRINGS[name]
+    except KeyError:
+        raise NotImplementedError(f"rotation pairing {name!r}: the kernels know {sorted(ROTATION_PAIRINGS)}") from None
+
+
 def qk_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cache,
-                       num_heads, num_kv_heads, head_dim, out_dtype=None) -> torch.Tensor:
+                       num_heads, num_kv_heads, head_dim, out_dtype=None, pairing: str = "halves") -> torch.Tensor:
     """From ``qkv [T, (Hq + 2 Hkv) D]`` (a tensor, or a ``SplitSum`` of it): per-head RMSNorm of q and k
-    (if weights are given), rotation of the first ``rope.shape[1]`` elements of each head by the angles
+    (if weights are given), rotation of the first ``rope.shape[1]`` elements of each head, in pairs as
+    ``pairing`` names them, by the angles
     of ``rope`` (a ``rope_table`` of these tokens; None: no rotation), k and v stored into the cache
     pages at ``slots`` (skipped when ``slots`` is None). Returns the tensor that holds the finished
     queries in its first ``Hq * D`` columns: ``qkv`` itself (written in place), or for a ``SplitSum`` a
@@ -464,7 +477,7 @@ def qk_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cac
         if slots.shape[0] != t:
             raise ValueError("one slot per token is needed")
         page_size = _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim)
-    rot_dim = 0
+    rot_dim, pair = 0, _pairing(pairing)
     if rope is not None:
         _dev(rope, "rope", F32, 2)
         rot_dim = rope.shape[1]
@@ -472,7 +485,7 @@ def qk_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cac
             raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
     _check(library().ms_qk_norm_rope_store(
         src, parts, splits, stride, q_out.data_ptr(), q_out.shape[1], int(dtype == BF16), _ptr(slots),
-        _ptr(q_weight), _ptr(k_weight), w_bf16, float(eps), _ptr(rope), int(rot_dim),
+        _ptr(q_weight), _ptr(k_weight), w_bf16, float(eps), _ptr(rope), int(rot_dim), pair,
         _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, t, num_heads,
         num_kv_heads, head_dim, page_size, _stream()), "qk_norm_rope_store")
     return q_out
@@ -503,12 +516,13 @@ def decode_splits(rows: int, num_kv_heads: int, max_kv_len: int) -> int:
     return max(1, min(by_fill, by_len))
 
 
-def decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim) -> bool:
+def decode_attention_fusable(qkv, batch, q_weight, k_weight, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
+                             pairing: str = "halves") -> bool:
     """Whether ``decode_attention_fused`` takes this step: every row brings one token, the qkv
     projection comes as partial sums, bfloat16 cache with 16-token pages, a head size of 64 or 128, at
-    most 16 query heads per KV head, bfloat16 norm weights (or none), rotation over the whole head (or
-    none)."""
-    return (isinstance(qkv, SplitSum) and batch.is_decode and batch.decode_tokens is None
+    most 16 query heads per KV head, bfloat16 norm weights (or none), rotation over the whole head in
+    pairs (j, j + D/2) (or none)."""
+    return (isinstance(qkv, SplitSum) and (rope is None or pairing == "halves") and batch.is_decode and batch.decode_tokens is None
             and k_cache.dtype == BF16 and v_cache.dtype == BF16 and k_cache.dim() == 4 and k_cache.shape[2] == 16
             and head_dim in (64, 128) and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16
             and qkv.stride % 4 == 0
@@ -572,7 +586,8 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
             merged = torch.empty((out_splits, t, n), dtype=F32, device=dev)
     out = None if merged is not None else torch.empty((t, num_heads * head_dim), dtype=BF16, device=dev)
     _check(lib.ms_attention_decode_fused_bf16(
-        qkv.parts.data_ptr(), qkv.splits, qkv.stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(rope), int(bool(store)),
+        qkv.parts.data_ptr(), qkv.splits, qkv.stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(rope),
+        ROTATION_PAIRINGS["halves"], int(bool(store)),
         k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], None,
         batch.token_row.data_ptr(), batch.positions.data_ptr(), _ptr(out), _ptr(part_o), _ptr(part_ml), t, splits,
         num_heads, num_kv_heads, head_dim, page, float(scale), int(window), int(merged is None), _stream()),

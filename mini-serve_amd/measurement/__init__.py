@@ -2,6 +2,6 @@
 and range markers that let a profiler keep to the measured steps."""
 
 from .markers import measured_region, mark
-from .sidecar import GpuSampler, sample_gpu, sidecar
+from .sidecar import GpuMonitor, gpu_now, sidecar
 
-__all__ = ["GpuSampler", "sample_gpu", "sidecar", "measured_region", "mark"]
+__all__ = ["GpuMonitor", "gpu_now", "sidecar", "measured_region", "mark"]

@@ -19,6 +19,8 @@ def run_to_completion(engine, max_steps: int | None = None) -> dict:
     times = {Phase.DECODE: [], Phase.MIXED: [], Phase.PREFILL: []}
     rows = {Phase.DECODE: 0, Phase.MIXED: 0, Phase.PREFILL: 0}
     tokens = {Phase.DECODE: 0, Phase.MIXED: 0, Phase.PREFILL: 0}
+    flops = {Phase.DECODE: 0, Phase.MIXED: 0, Phase.PREFILL: 0}
+    step_flops = getattr(getattr(getattr(engine, "runner", None), "model", None), "step_flops", None)  # what the parts say a step costs
     steps = 0
     t0 = time.perf_counter()
     while engine.has_unfinished and (max_steps is None or steps < max_steps):
@@ -32,6 +34,8 @@ def run_to_completion(engine, max_steps: int | None = None) -> dict:
         times[batch.phase].append(t)
         rows[batch.phase] += len(batch.rows)
         tokens[batch.phase] += batch.num_tokens
+        if step_flops is not None:
+            flops[batch.phase] += step_flops([(n, s) for _, s, n in batch.rows])
     span = time.perf_counter() - t0
 
     def kind(p):
@@ -39,6 +43,7 @@ def run_to_completion(engine, max_steps: int | None = None) -> dict:
         if not ts:
             return {"steps": 0}
         return {"steps": len(ts), "median_ms": round(statistics.median(ts) * 1e3, 4), "mean_ms": round(sum(ts) / len(ts) * 1e3, 4),
-                "mean_rows": round(rows[p] / len(ts), 2), "mean_tokens": round(tokens[p] / len(ts), 2)}
+                "mean_rows": round(rows[p] / len(ts), 2), "mean_tokens": round(tokens[p] / len(ts), 2),
+                "mean_flops": flops[p] / len(ts)}
 
     return {"seconds": span, "steps": steps, "decode": kind(Phase.DECODE), "mixed": kind(Phase.MIXED), "prefill": kind(Phase.PREFILL)}

@@ -89,8 +89,9 @@ class GQAttention(Mixer):
         qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
         rot = self.position.rotation(batch)
         table = rot.table if rot is not None else None
+        pairing = rot.pairing if rot is not None else "halves"
         if ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
-                                        self.heads, self.kv_heads, self.head_dim):
+                                        self.heads, self.kv_heads, self.head_dim, pairing):
             # a step of single tokens: norm, rotation, cache store and attention are one kernel
             # ... and, with few rows, the reduction of the key splits and the output projection another
             out = ops.decode_attention_fused(
@@ -105,7 +106,7 @@ class GQAttention(Mixer):
             qkv, cache.slots if cache.writes else None,
             self.q_norm, self.k_norm, 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps),
             table,
-            cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, out_dtype=self.rt.dtype,
+            cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, out_dtype=self.rt.dtype, pairing=pairing,
         )
         out = ops.paged_attention(
             q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
@@ -116,3 +117,17 @@ class GQAttention(Mixer):
     def parameters_bytes(self) -> int:
         ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else [])
         return sum(t.numel() * t.element_size() for t in ts)
+
+    def flops(self, rows) -> int:
+        """The four projections, and both attention products over every (query, visible key) pair: a query
+        at position p sees keys ``max(0, p - window + 1) .. p``."""
+        tokens = sum(n for n, _ in rows)
+        pairs = 0
+        for n, cached in rows:
+            for p in (range(cached, cached + n) if self.window else ()):
+                pairs += min(p + 1, self.window)
+            if not self.window:
+                pairs += n * cached + n * (n + 1) // 2
+        width = self.heads * self.head_dim
+        linear = 2 * tokens * self.hidden * (width + 2 * self.kv_heads * self.head_dim) + 2 * tokens * width * self.hidden
+        return linear + 4 * pairs * width

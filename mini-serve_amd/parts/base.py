@@ -120,11 +120,14 @@ class StateNeed:
 @dataclass(frozen=True)
 class Rotation:
     """Rotary position encoding as a mixer's kernels need it: the first ``dim`` elements of each
-    head are turned in pairs (j, j + dim/2) by the step's angles, whose cosines and sines are the two
-    halves of a row of ``table``."""
+    head are turned in pairs by the step's angles, whose cosines and sines are the two halves of a row
+    of ``table`` (pair ``j`` by angle ``j``). ``pairing`` says which elements make pair ``j``:
+    ``"halves"`` (j, j + dim/2), ``"adjacent"`` (2j, 2j + 1); the kernels name the pairings they know
+    (``ops.ROTATION_PAIRINGS``) and refuse any other."""
 
     dim: int
     table: Any  # float32 device tensor [tokens of the step, dim]: cosines, then sines
+    pairing: str = "halves"
 
 
 class Runtime:
@@ -151,11 +154,24 @@ class Part:
         for parts outside layers)."""
         return {}
 
+    @classmethod
+    def aliases(cls, spec: PartSpec) -> dict[str, str]:
+        """Tensors this part reads that are stored under another name: ``{name: source}``, ``name``
+        relative like the names of ``tensors`` (and never among them), ``source`` the full name of a
+        tensor some part declares. The part receives the source's tensor under ``name`` (the same memory,
+        no copy); a tensor stored under ``name`` itself is a duplicate and is dropped."""
+        return {}
+
     def bind(self, tensors: Mapping[str, "torch.Tensor"]) -> None:
-        """Receive the tensors declared by ``tensors`` (same names), already on the device."""
+        """Receive the tensors declared by ``tensors`` and ``aliases`` (same names), already on the device."""
 
     def parameters_bytes(self) -> int:
         """Bytes of weights a decode step reads from this part (for the bandwidth model)."""
+        return 0
+
+    def flops(self, rows) -> int:
+        """Floating-point operations of one pass over ``rows``: a list of ``(new tokens, tokens already in
+        the cache)`` per request; a multiply-add counts two. What a measurement divides by its time."""
         return 0
 
 

@@ -51,11 +51,18 @@ class LinearHead(Head):
             return {}
         return {spec["tensor"]: TensorSpec((int(spec["vocab_size"]), int(spec["width"])))}
 
+    @classmethod
+    def aliases(cls, spec: PartSpec) -> dict[str, str]:
+        return {spec["tensor"]: spec["tied_to"]} if spec.get("tied_to") else {}
+
     def bind(self, tensors) -> None:
-        self.weight = tensors[self.tied_to or self.spec["tensor"]]
+        self.weight = tensors[self.spec["tensor"]]
 
     def forward(self, x):
         return self.rt.ops.linear(x, self.weight, out_dtype=torch.float32)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
+
+    def flops(self, rows) -> int:
+        return 2 * len(rows) * self.vocab * self.width  # one wanted position per request

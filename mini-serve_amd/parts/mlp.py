@@ -53,3 +53,6 @@ class GatedMLP(FeedForward):
 
     def parameters_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.gate_up, self.down))
+
+    def flops(self, rows) -> int:
+        return 2 * sum(n for n, _ in rows) * 3 * self.hidden * self.inter

@@ -35,6 +35,30 @@ def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
     return out
 
 
+def expected_aliases(spec: ModelSpec) -> dict[str, str]:
+    """Every tensor name a part reads under which nothing is stored, with the full name of the tensor
+    that stands for it, collected from the parts' own ``aliases``. A source must be a declared tensor."""
+    out: dict[str, str] = {}
+
+    def add(aliases: dict[str, str], prefix: str = "") -> None:
+        for name, source in aliases.items():
+            out[prefix + name] = source
+
+    add(part_class("embedding", spec.embedding).aliases(spec.embedding))
+    for layer in spec.layers:
+        for category, part in (("block", layer.block), ("mixer", layer.mixer), ("feed_forward", layer.feed_forward)):
+            add(part_class(category, part).aliases(part), layer.prefix)
+    add(part_class("norm", spec.final_norm).aliases(spec.final_norm))
+    add(part_class("head", spec.head).aliases(spec.head))
+    declared = expected_tensors(spec)
+    for name, source in out.items():
+        if name in declared:
+            raise ValueError(f"tensor {name} is declared as stored and as an alias of {source}")
+        if source not in declared:
+            raise ValueError(f"tensor {name} is an alias of {source}, which no part declares")
+    return out
+
+
 @dataclass(frozen=True)
 class CacheSlotNeed:
     """What one cache slot of the run order holds: paged keys/values and/or fixed-size state."""
@@ -52,7 +76,12 @@ class DecoderModel:
         self.device = rt.device
         self.vocab_size = spec.vocab_size
 
-        def local(prefix: str, names) -> dict:
+        weights = dict(weights)
+        for name, source in expected_aliases(spec).items():
+            weights[name] = weights[source]  # the same tensor under its second name
+
+        def local(prefix: str, part_type, part_spec) -> dict:
+            names = list(part_type.tensors(part_spec)) + list(part_type.aliases(part_spec))
             return {n: weights[prefix + n] for n in names}
 
         self.embedding = part_class("embedding", spec.embedding)(spec.embedding, rt)
@@ -60,11 +89,11 @@ class DecoderModel:
         self.blocks = []
         for layer in spec.layers:
             mixer = part_class("mixer", layer.mixer)(layer.mixer, rt)
-            mixer.bind(local(layer.prefix, type(mixer).tensors(layer.mixer)))
+            mixer.bind(local(layer.prefix, type(mixer), layer.mixer))
             ffn = part_class("feed_forward", layer.feed_forward)(layer.feed_forward, rt)
-            ffn.bind(local(layer.prefix, type(ffn).tensors(layer.feed_forward)))
+            ffn.bind(local(layer.prefix, type(ffn), layer.feed_forward))
             block = part_class("block", layer.block)(layer.block, rt, mixer, ffn)
-            block.bind(local(layer.prefix, type(block).tensors(layer.block)))
+            block.bind(local(layer.prefix, type(block), layer.block))
             self.blocks.append(block)
         self.final_norm = part_class("norm", spec.final_norm)(spec.final_norm, rt)
         self.final_norm.bind(weights)
@@ -109,6 +138,15 @@ class DecoderModel:
             return None
         x = self.final_norm.forward(residual, rows=batch.want_rows, add=pending)
         return self.head.forward(x)
+
+    def step_flops(self, rows) -> int:
+        """Floating-point operations of one step over ``rows`` (``(new tokens, cached tokens)`` per request),
+        logits at one position per request: the sum of what the parts say of themselves."""
+        total = self.final_norm.flops(rows) + self.head.flops(rows)
+        for e in self.spec.run_order:
+            b = self.blocks[e.layer]
+            total += b.flops(rows) + b.mixer.flops(rows) + b.feed_forward.flops(rows)
+        return total
 
     def decode_read_bytes(self) -> int:
         """Bytes of weights one decode step reads: every run-order entry's layer once, the final

@@ -1,4 +1,4 @@
-from .loader import WeightsError, load_weights, tied_names
+from .loader import WeightsError, load_weights
 from .random_init import Init, random_tensors, write_model_folder
 
-__all__ = ["WeightsError", "load_weights", "tied_names", "Init", "random_tensors", "write_model_folder"]
+__all__ = ["WeightsError", "load_weights", "Init", "random_tensors", "write_model_folder"]

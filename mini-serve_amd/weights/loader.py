@@ -8,8 +8,9 @@ wrong or partial checkpoint fails at load and never inside a forward pass (:121-
 Dtypes: with compute dtype bfloat16, 16-bit float tensors are kept in bfloat16 and a tensor stored
 in 32-bit stays 32-bit (the part that owns it then computes with it in 32-bit); with compute
 dtype float32 every float tensor is widened to float32 (exact). Integer tables become int32.
-A tied head gets no tensor of its own: a duplicate ``lm_head.weight`` in the file is dropped and
-the head reads the embedding's tensor (:116-119,135-136).
+A part may read a tensor under a second name (``Part.aliases``: a tied head reads the embedding's
+table as its own weight, :116-119,135-136): nothing is stored for that name, a duplicate in the file is
+dropped, and the name maps to the source's tensor itself.
 """
 
 from __future__ import annotations
@@ -20,7 +21,7 @@ import torch
 from safetensors import safe_open
 
 from ..config.spec import ModelSpec
-from ..parts.model import expected_tensors
+from ..parts.model import expected_aliases, expected_tensors
 
 _FLOAT16 = (torch.bfloat16, torch.float16)
 MAX_LISTED = 8
@@ -56,12 +57,6 @@ def _place(t: torch.Tensor, kind: str, dtype: torch.dtype) -> torch.Tensor:
     return t.to(torch.float32)  # stored in 32-bit (or wider): stays 32-bit
 
 
-def tied_names(spec: ModelSpec) -> dict[str, str]:
-    """Tensor names that alias another tensor instead of being stored: ``{alias: source}``."""
-    tied = spec.head.get("tied_to")
-    return {spec.head["tensor"]: tied} if tied else {}
-
-
 def load_weights(
     path: str | Path,
     spec: ModelSpec,
@@ -75,7 +70,7 @@ def load_weights(
     if not files:
         raise FileNotFoundError(f"no .safetensors files in {path}")
     want = expected_tensors(spec)
-    aliases = tied_names(spec)
+    aliases = expected_aliases(spec)  # names the parts read another tensor under: nothing is stored for them
 
     weights: dict[str, torch.Tensor] = {}
     unexpected: list[str] = []
@@ -100,4 +95,6 @@ def load_weights(
     missing = sorted(want.keys() - weights.keys() - {m.split(":")[0] for m in mismatched})
     if missing or unexpected or mismatched:
         raise WeightsError(path, missing, sorted(unexpected), sorted(mismatched))
+    for name, source in aliases.items():
+        weights[name] = weights[source]
     return weights

@@ -313,3 +313,51 @@ def test_default_pool_is_sized_from_a_measured_peak(folders):
     assert [len(g) for g in got] == [6, 6] and eng.runner.cache.idle
     with pytest.raises(ValueError, match="fit in memory"):
         engine(folders["tinyD"], "bfloat16", kv_pool_tokens=2**40)
+
+
+def test_a_windowed_group_gets_the_pages_it_can_use_and_the_rest_goes_to_the_others(folders):
+    """tinyE keeps every key in two layers and a window of 100 in one. With prompts cut into portions of 64 a
+    request never holds more than the window and a portion in the windowed layer: that group gets
+    ``max_running * (pages(window - 1 + portion) + 1)`` pages, whether the pool is given in tokens or measured,
+    and a measured pool spends what that saves on the other group. Generation is unchanged."""
+    from miniserve_amd.engine.describe import engine_description
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, w = read_model_folder(folders["tinyE"])
+    need = 4 * (-(-(100 - 1 + 64) // 16) + 1)
+    eng = engine(folders["tinyE"], "bfloat16", max_running=4, chunked_prefill_size=64, kv_pool_tokens=4096)
+    assert [(g.window, n) for g, n in zip(eng.runner.layout.groups, eng.runner.cache.total_pages())] == [(0, 256), (100, need)]
+    d = engine_description(eng)
+    assert d["kv_pool_pages"] == [256, need] and d["kv_profile"]["pages_per_group"] == [256, need]
+    prompts = prompts_for(cfg, [300, 40, 7])
+    want = [P.greedy(cfg, w, p, 6) for p in prompts]
+    ref = engine(folders["tinyE"], "float32", max_running=4, chunked_prefill_size=64, kv_pool_tokens=4096)
+    assert ref.generate(prompts, SamplingParams(max_new_tokens=6)) == want and ref.runner.cache.idle
+    del ref
+    measured = engine(folders["tinyE"], "bfloat16", max_running=4, chunked_prefill_size=64, kv_mem_fraction=0.01)
+    prof = measured.runner.kv_profile
+    per_group = measured.runner.layout.bytes_per_page(16, 2)
+    budget = int(0.01 * (prof["free_bytes"] - prof["peak_activation_bytes"] - prof["graph_reserve_bytes"]))
+    assert prof["pages_per_group"] == [(budget - need * per_group[1]) // per_group[0], need]
+    got = measured.generate(prompts, SamplingParams(max_new_tokens=6))
+    assert [len(g) for g in got] == [6, 6, 6] and measured.runner.cache.idle
+    # whole prompts run in one step however long: no bound on what the windowed group holds, it is sized like the other
+    whole = engine(folders["tinyE"], "bfloat16", max_running=4, chunked_prefill_size=0, kv_pool_tokens=4096)
+    assert whole.runner.cache.total_pages() == [256, 256]
+
+
+def test_a_measured_pool_refuses_whole_prompts_beyond_the_step_it_was_measured_with(folders):
+    """Whole prompts run in one step. A pool sized from the measured peak of a step of ``max_prefill_tokens`` tokens
+    leaves no room for the activations of a longer step, so such a prompt is refused at submission; with a pool
+    given in tokens nothing was measured and the prompt runs."""
+    from miniserve_amd.engine.request import SamplingParams
+
+    cfg, _ = read_model_folder(folders["tinyD"])
+    long_prompt = prompts_for(cfg, [300])[0]
+    eng = engine(folders["tinyD"], "bfloat16", max_running=2, chunked_prefill_size=0, max_prefill_tokens=128, kv_mem_fraction=0.01)
+    assert eng.runner.kv_profile["profile_tokens"] == 128
+    with pytest.raises(ValueError, match="use chunked prefill"):
+        eng.add_request(long_prompt, SamplingParams(max_new_tokens=4))
+    assert len(eng.generate([long_prompt[:100]], SamplingParams(max_new_tokens=4))[0]) == 4
+    given = engine(folders["tinyD"], "bfloat16", max_running=2, chunked_prefill_size=0, max_prefill_tokens=128, kv_pool_tokens=1024)
+    assert len(given.generate([long_prompt], SamplingParams(max_new_tokens=4))[0]) == 4

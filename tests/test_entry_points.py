@@ -60,11 +60,51 @@ def test_bench_line_on_a_tiny_shape():
     assert set(line["roofline"]) == {"bound", "achieved", "peak", "unit", "frac"} and line["roofline"]["peak"] == 8000.0
     assert line["prefill"]["tokens"] == 128 and line["prefill"]["value"] > 0
     assert set(line["points"]) == {"decode_b1", "decode_b1_frac", "decode_b64", "decode_b64_frac"}
-    assert line["config"]["warmup_steps_run"] == 20  # at least --warmup steps and --warmup-seconds at a millisecond a step
+    assert line["config"]["warmup_steps_run"] == 2
     side = line["sidecar"]
     assert side["runtime"]["torch"] and side["runtime"]["kernel_library"].startswith("libmsamd_kernels_")
     assert side["engine"]["kv_pool_tokens"] == [2 * (512 + 32)] * 2 and side["engine"]["decode_graph"] is True
-    assert side["engine"]["chunked_prefill_size"] == 2048 and side["warmup"]["steps"] == 20
+    assert side["engine"]["chunked_prefill_size"] == 2048 and side["warmup"]["steps"] == 2
+    # after the warm-up steps the last one is repeated, at least for the time asked for and until the clock is steady
+    assert side["warmup"]["repeats_of_the_last_step"] >= 8 and side["warmup"]["held_seconds"] >= 0.02
+    assert side["warmup"]["clock_steady"] in (True, False, None)
+    assert "copy_GBps" in line["measured_peaks"] and line["measured_peaks"]["copy_GBps"] > 100
+    assert side["conditions"]["power_limit_w"] is None or 100 < side["conditions"]["power_limit_w"] < 5000
+
+
+@pytest.mark.gpu
+def test_the_monitor_reads_a_loaded_gpu():
+    """The readings themselves, not their arithmetic: under a sustained matrix product the shader clock is
+    far above its idle value, the socket draws a plausible power (a scale wrong by a thousand shows), the
+    memory clock and the temperatures are there, and the limits name a power limit above what is drawn."""
+    import time
+
+    import torch
+
+    from miniserve_amd.kernels import ops
+    from miniserve_amd.measurement import GpuMonitor
+
+    x = torch.randn((8192, 8192), device="cuda:0").to(torch.bfloat16)
+    w = torch.randn((8192, 8192), device="cuda:0").to(torch.bfloat16)
+
+    def work():
+        for _ in range(10):
+            ops.linear(x, w, out_dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+
+    with GpuMonitor(interval_s=0.02) as g:
+        t0 = time.monotonic()
+        out = g.warm_until_steady(work, least_s=1.0, most_s=4.0)
+        busy = g.window(since=t0 + 0.5)
+        limits = g.conditions()
+    assert out["steady"] is not None, "the clock could be read often enough to decide"
+    assert busy["samples"] >= 10
+    assert busy["sclk_mhz"]["mean"] > 1000, busy
+    assert 50 < busy["power_w"]["mean"] < 2000 and busy["power_w"]["max"] < 2000, busy
+    assert busy["mclk_mhz"]["mean"] > 500 and 10 < busy["temp_c"]["mean"] < 120, busy
+    assert busy["busy_pct"]["max"] > 50, busy
+    assert limits["power_limit_w"] is not None and limits["power_limit_w"] >= busy["power_w"]["mean"] * 0.9, limits
+    assert limits["sclk_range_mhz"] is not None and limits["sclk_range_mhz"][1] >= busy["sclk_mhz"]["max"] * 0.95
 
 
 @pytest.mark.gpu

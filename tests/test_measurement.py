@@ -8,60 +8,111 @@ import itertools
 
 import pytest
 
-from miniserve_amd.measurement import GpuSampler, mark, measured_region, sample_gpu
+import time
+
+import numpy as np
+
+from miniserve_amd.measurement import GpuMonitor, gpu_now, mark, measured_region
 from miniserve_amd.measurement.offline import run_to_completion
+from miniserve_amd.measurement.sidecar import COLUMNS, throttled_share
 
 
 def readings(clocks, power=None, t0=100.0, dt=0.1):
-    return [{"t": t0 + i * dt, "sclk_mhz": c, "power_w": None if power is None else power[i], "temp_c": 40.0, "util_pct": 99.0}
-            for i, c in enumerate(clocks)]
+    """Rows in the monitor's column order: time, shader clock, memory clock, power, two temperatures, two activities."""
+    return [(t0 + i * dt, c, 2000.0, None if power is None else power[i], 40.0, 35.0, 99.0, 10.0) for i, c in enumerate(clocks)]
+
+
+def monitor_with(rows, **kw):
+    g = GpuMonitor(**kw)
+    g.load(rows)
+    return g
 
 
 def test_a_reading_without_a_gpu_says_unknown_not_zero():
-    s = sample_gpu()
-    assert set(s) == {"t", "sclk_mhz", "power_w", "temp_c", "util_pct"} and s["t"] > 0
-    assert all(s[k] is None or s[k] >= 0 for k in ("sclk_mhz", "power_w", "temp_c", "util_pct"))
+    s = gpu_now()
+    assert set(s) == set(COLUMNS[1:]) and "power_w" in s and "mclk_mhz" in s
+    assert all(v is None or v >= 0 for v in s.values())
 
 
-def test_the_clock_has_settled_when_two_windows_agree():
-    g = GpuSampler()
-    g.samples = readings([2400, 2400, 2400])
-    assert g.settled() is None, "fewer than two windows of readings decide nothing"
-    g.samples = readings([2400, 2300, 2100, 1900, 1750, 1720, 1700, 1700])  # still falling: 2175 against 1717
-    assert g.settled() is False
-    g.samples = readings([2400, 2300, 2100, 1900, 1710, 1700, 1705, 1695, 1700, 1702, 1698, 1700])
-    assert g.settled() is True  # the last four against the four before them: within 2 %
-    g.samples = readings([1700] * 4 + [1740] * 4)  # 2.3 % apart
-    assert g.settled() is False and g.settled(tol=0.03) is True
-    g.samples = readings([None] * 20)
-    assert g.settled() is None, "a clock that cannot be read settles nothing"
-    g.samples = readings([1700, None, 1700, 1700, None, 1700, 1700, 1700, 1700, 1700])  # unknown readings are skipped
-    assert g.settled() is True
+def test_the_clock_is_steady_when_two_runs_of_readings_agree():
+    assert monitor_with(readings([2400, 2400, 2400])).steady(readings=4) is None, "fewer than two runs of readings decide nothing"
+    falling = monitor_with(readings([2400, 2300, 2100, 1900, 1750, 1720, 1700, 1700]))  # 2175 against 1717
+    assert falling.steady(readings=4) is False
+    flat = monitor_with(readings([2400, 2300, 2100, 1900, 1710, 1700, 1705, 1695, 1700, 1702, 1698, 1700]))
+    assert flat.steady(readings=4) is True  # the last four against the four before them: within 2 %
+    step = monitor_with(readings([1700] * 4 + [1740] * 4))  # 2.3 % apart
+    assert step.steady(readings=4) is False and step.steady(readings=4, tolerance=0.03) is True
+    assert monitor_with(readings([None] * 20)).steady() is None, "a clock that cannot be read settles nothing"
+    gaps = monitor_with(readings([1700, None, 1700, 1700, None, 1700, 1700, 1700, 1700, 1700]))  # unknown readings are skipped
+    assert gaps.steady(readings=4) is True
 
 
-def test_the_summary_covers_the_timed_window_only():
-    g = GpuSampler()
-    g.samples = readings([2400, 2000, 1800, 1700, 1700, 2400], power=[100, 600, 900, 1000, 1000, 120])
-    whole = g.summary()
+def test_the_window_covers_the_timed_span_only():
+    g = monitor_with(readings([2400, 2000, 1800, 1700, 1700, 2400], power=[100, 600, 900, 1000, 1000, 120]))
+    whole = g.window()
     assert whole["samples"] == 6 and whole["sclk_mhz"] == {"min": 1700, "max": 2400, "mean": 2000.0}
-    inside = g.summary(since=100.15, until=100.45)  # readings 2, 3 and 4
+    inside = g.window(since=100.15, until=100.45)  # readings 2, 3 and 4
     assert inside["samples"] == 3 and inside["sclk_mhz"] == {"min": 1700, "max": 1800, "mean": 1733.3}
-    assert inside["power_w"] == {"min": 900, "max": 1000, "mean": 966.7}
-    assert g.summary(since=200.0) == {"samples": 0, "sclk_mhz": None, "power_w": None, "temp_c": None}
-    g.samples = readings([None, None])
-    assert g.summary()["sclk_mhz"] is None and g.summary()["temp_c"]["mean"] == 40.0
+    assert inside["power_w"] == {"min": 900, "max": 1000, "mean": 966.7} and inside["mclk_mhz"]["mean"] == 2000.0
+    empty = g.window(since=200.0)
+    assert empty["samples"] == 0 and all(empty[c] is None for c in COLUMNS[1:])
+    g = monitor_with(readings([None, None]))
+    assert g.window()["sclk_mhz"] is None and g.window()["temp_c"]["mean"] == 40.0
 
 
-def test_the_sampler_thread_collects_and_stops():
-    with GpuSampler(interval_s=0.01) as g:
-        first = g.sample_now()
-        while len(g.snapshot()) < 3:
+def test_the_ring_keeps_the_latest_readings_in_order():
+    g = monitor_with(readings(range(1000, 1010)), capacity=4)
+    assert g.column("sclk_mhz").tolist() == [1006, 1007, 1008, 1009]
+    assert np.all(np.diff(g.column("t")) > 0)
+
+
+def test_the_monitor_thread_collects_and_stops():
+    with GpuMonitor(interval_s=0.01) as g:
+        first = g.read_now()
+        while len(g.readings()) < 3:
             pass
-    n = len(g.snapshot())
-    assert n >= 3 and first in [s["t"] for s in g.snapshot()]
-    times = [s["t"] for s in g.snapshot()]
-    assert times == sorted(times)
-    assert len(g.snapshot()) == n, "no reading after the with block has ended"
+    n = len(g.readings())
+    times = g.column("t")
+    assert n >= 3 and first in times and np.all(np.diff(times) >= 0)
+    time.sleep(0.03)
+    assert len(g.readings()) == n, "no reading after the with block has ended"
+
+
+def test_warming_waits_for_a_steady_clock_between_a_least_and_a_most_time():
+    """``work`` stands for a few decode steps; the readings are fed by the test instead of a thread."""
+    g = GpuMonitor()
+    clocks = iter([2400, 2300, 2200, 2100, 2000, 1900, 1800] + [1700] * 200)
+
+    def work():
+        g._append([time.monotonic(), next(clocks), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0])
+        time.sleep(0.004)
+
+    out = g.warm_until_steady(work, least_s=0.02, most_s=2.0, readings=3)
+    # falling for seven readings, then flat: steady once the last three and the three before them agree
+    assert out["steady"] is True and 0.02 <= out["seconds"] < 1.0 and 10 <= out["calls"] < 100
+    falling = iter(range(2400, 0, -20))
+    g2 = GpuMonitor()
+
+    def cooling():
+        g2._append([time.monotonic(), next(falling), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0])
+        time.sleep(0.004)
+
+    out = g2.warm_until_steady(cooling, least_s=0.01, most_s=0.15, readings=3)
+    assert out["steady"] is False and out["seconds"] >= 0.15, "a clock that keeps moving ends the wait at the most time, and says so"
+    g3 = GpuMonitor()
+    out = g3.warm_until_steady(lambda: time.sleep(0.002), least_s=0.01, most_s=0.03)
+    assert out["steady"] is None and out["seconds"] >= 0.03, "a clock that cannot be read decides nothing"
+    stale = monitor_with(readings([1700] * 40, t0=time.monotonic() - 100))
+    out = stale.warm_until_steady(lambda: time.sleep(0.002), least_s=0.01, most_s=0.03)
+    assert out["steady"] is None, "readings from before the warm-up do not count"
+
+
+def test_the_share_of_time_held_back_is_a_difference_of_counters():
+    before = {"all": 1000.0, "power": 100.0, "socket_temperature": 0.0, "hot_spot": 0.0, "regulator_temperature": 0.0, "memory_temperature": float("nan")}
+    after = {"all": 3000.0, "power": 600.0, "socket_temperature": 0.0, "hot_spot": 20.0, "regulator_temperature": 0.0, "memory_temperature": float("nan")}
+    share = throttled_share(before, after)
+    assert share == {"power": 0.25, "socket_temperature": 0.0, "hot_spot": 0.01, "regulator_temperature": 0.0, "memory_temperature": None}
+    assert throttled_share(None, after) is None and throttled_share(before, before) is None  # the counter did not run
 
 
 def test_markers_do_nothing_outside_a_profiler():

@@ -167,9 +167,11 @@ def test_embedding_and_head_alone(dtype):
         h_spec = PartSpec("linear_head", {"vocab_size": 301, "width": 40, "tensor": "lm", "tied_to": tied})
         head = part_class("head", h_spec)(h_spec, rt)
         w = tensor((301, 40), rt, 2)
-        head.bind({"E": table, "lm": w})
-        assert (head.weight is table) == (tied is not None)
+        # a tied head declares no tensor of its own but an alias: it is handed the source under its own name
+        assert type(head).aliases(h_spec) == ({"lm": "E"} if tied else {})
         assert type(head).tensors(h_spec) == ({} if tied else {"lm": type(head).tensors(h_spec)["lm"]})
+        head.bind({"lm": table if tied else w})
+        assert (head.weight is table) == (tied is not None)
         x = tensor((3, 40), rt, 3)
         logits = head.forward(x)
         assert logits.dtype == torch.float32

@@ -29,7 +29,7 @@ def test_round_trip_and_tied_head(tmp_path):
     folder = write_model_folder(tmp_path / "m", REF_TINY, seed=0)
     spec = spec_of(REF_TINY)
     w = load_weights(folder, spec, torch.bfloat16, "cpu")
-    assert "lm_head.weight" not in w  # the head reads the embedding's tensor itself
+    assert w["lm_head.weight"] is w["model.embed_tokens.weight"]  # the head reads the embedding's tensor itself
     assert all(t.dtype == torch.bfloat16 for t in w.values())
     again = random_tensors(spec, 0)
     assert all(torch.equal(w[k], again[k]) for k in again)
@@ -45,7 +45,51 @@ def test_a_duplicate_head_in_a_tied_checkpoint_is_dropped(tmp_path):
     t = load_file(str(folder / "model.safetensors"))
     t["lm_head.weight"] = torch.zeros(32, 8, dtype=torch.bfloat16)
     save_file(t, str(folder / "model.safetensors"))
-    assert "lm_head.weight" not in load_weights(folder, spec_of(REF_TINY), torch.bfloat16, "cpu")
+    w = load_weights(folder, spec_of(REF_TINY), torch.bfloat16, "cpu")
+    assert w["lm_head.weight"] is w["model.embed_tokens.weight"] and float(w["lm_head.weight"].float().abs().max()) > 0
+
+
+def test_the_loader_follows_whatever_aliases_the_parts_declare(tmp_path):
+    """Not the head's private affair: a feed-forward defined here reads a norm weight of another layer under a
+    name of its own. Nothing is stored for that name, a stored duplicate is dropped, the name maps to the
+    source's tensor itself; an alias of something no part declares is an error when the model is described."""
+    import dataclasses
+
+    from miniserve_amd.config import PartSpec
+    from miniserve_amd.parts import FeedForward, TensorSpec, register, unregister
+    from miniserve_amd.parts.model import expected_aliases, expected_tensors
+
+    @register("feed_forward", "test_scaled")
+    class Scaled(FeedForward):
+        @classmethod
+        def tensors(cls, spec):
+            return {"ff.weight": TensorSpec((8, 8))}
+
+        @classmethod
+        def aliases(cls, spec):
+            return {"ff.scale": spec["scale_from"]}
+
+    try:
+        spec = spec_of(REF_TINY)
+        layers = list(spec.layers)
+        layers[1] = dataclasses.replace(layers[1], feed_forward=PartSpec("test_scaled", {"scale_from": "model.layers.0.input_layernorm.weight"}))
+        spec = dataclasses.replace(spec, layers=tuple(layers))
+        assert expected_aliases(spec) == {"model.layers.1.ff.scale": "model.layers.0.input_layernorm.weight",
+                                          "lm_head.weight": "model.embed_tokens.weight"}
+        assert "model.layers.1.ff.scale" not in expected_tensors(spec)
+        tensors = random_tensors(spec, 3, Init(0.05, (0.5, 1.5)))
+        assert "model.layers.1.ff.scale" not in tensors
+        tensors["model.layers.1.ff.scale"] = torch.zeros(8, dtype=torch.bfloat16)  # a duplicate under the alias: dropped
+        folder = tmp_path / "m"
+        folder.mkdir()
+        save_file(tensors, str(folder / "model.safetensors"))
+        w = load_weights(folder, spec, torch.bfloat16, "cpu")
+        assert w["model.layers.1.ff.scale"] is w["model.layers.0.input_layernorm.weight"]
+        bad = dataclasses.replace(spec, layers=(layers[0], dataclasses.replace(layers[1], feed_forward=PartSpec("test_scaled", {"scale_from": "nowhere.weight"}))))
+        with pytest.raises(ValueError, match="nowhere.weight"):
+            expected_aliases(bad)
+    finally:
+        unregister("feed_forward", "test_scaled")
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
