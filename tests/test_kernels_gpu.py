@@ -394,6 +394,53 @@ def test_qk_norm_rope_store(ops, dtype, hq, hkv, d, rot, page, t, layout):
     close(kc2.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)[sl], kn, tol, "k from partial sums")
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("hq,hkv,d,rot", [(4, 2, 16, 16), (3, 1, 64, 64), (16, 8, 128, 128), (5, 5, 48, 20), (2, 1, 256, 64)])
+def test_qk_norm_rope_store_turns_adjacent_elements(ops, dtype, hq, hkv, d, rot):
+    """The other pairing: elements (2j, 2j + 1) of a head are turned by angle j. Head sizes 64 and 128 take the
+    wave-per-head kernel here too (the tiled one knows halves only); a pairing no kernel knows is refused."""
+    t, page, eps = 70, 16, 1e-5
+    pages = t // page + 3
+    qkv = rand((t, (hq + 2 * hkv) * d), dtype, 26)
+    qw, kw = rand((d,), dtype, 27) + 1, rand((d,), dtype, 28) + 1
+    pos = torch.tensor(([0, 1, 2, 3, 40, 41, 700, 5, 6, 4000] * 7)[:t], dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * page, generator=torch.Generator().manual_seed(2))[:t].to(torch.int32).to(DEV)
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    rope = ops.rope_table(pos, inv_freq)
+    kc, vc = torch.zeros((pages, hkv, page, d), dtype=dtype, device=DEV), torch.zeros((pages, hkv, d, page), dtype=dtype, device=DEV)
+    ref = qkv.double().view(t, hq + 2 * hkv, d)
+
+    def norm(x, w):
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
+
+    def turn(x):
+        ang = (pos.float()[:, None] * inv_freq[None, :]).double()
+        cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        out = x.clone()
+        a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+        out[..., 0:rot:2], out[..., 1:rot:2] = a * cos - b * sin, b * cos + a * sin
+        return out
+
+    work = qkv.clone()
+    ops.qk_norm_rope_store(work, slots, qw, kw, eps, rope, kc, vc, hq, hkv, d, pairing="adjacent")
+    tol = 2e-6 if dtype == F32 else 5e-3
+    close(work.view(t, hq + 2 * hkv, d)[:, :hq], turn(norm(ref[:, :hq], qw)), tol, "q, adjacent pairs")
+    got_k = kc.permute(0, 2, 1, 3).reshape(pages * page, hkv, d)
+    close(got_k[slots.long()], turn(norm(ref[:, hq : hq + hkv], kw)), tol, "k in cache, adjacent pairs")
+    if rot == d:  # and it is another rotation than that of the halves
+        halves = qkv.clone()
+        ops.qk_norm_rope_store(halves, slots, qw, kw, eps, rope, torch.zeros_like(kc), torch.zeros_like(vc), hq, hkv, d)
+        assert float((halves.float() - work.float()).abs().max()) > 0.1
+    with pytest.raises(NotImplementedError, match="pairing"):
+        ops.qk_norm_rope_store(work, slots, qw, kw, eps, rope, kc, vc, hq, hkv, d, pairing="quarters")
+    # the fused decode step takes halves only and says so
+    batch = make_batch([1] * t, pos.tolist())
+    parts = ops.SplitSum(torch.stack([qkv.float()]))
+    if dtype == BF16 and d in (64, 128) and rot == d:
+        assert ops.decode_attention_fusable(parts, batch, qw, kw, rope, kc, vc, hq, hkv, d)
+        assert not ops.decode_attention_fusable(parts, batch, qw, kw, rope, kc, vc, hq, hkv, d, "adjacent")
+
+
 class _Batch:
     def prefill_tiles(self, tile_tokens):
         from miniserve_amd.kernels.ops import build_prefill_tiles
