@@ -17,10 +17,11 @@ One JSON line is printed. ``value`` = decoded tokens per second of the headline 
 of themselves), ``roofline`` (the decode step's bytes,
 every weight once plus the live requests' cache, over its time, against the published 8 TB/s),
 ``points`` (decode at batch 1 and 64 of the same shape; unless ``--no-extra``, decode at batch 8 behind
-32,768 tokens and a prompt of 8,192 tokens in one step, the Qwen3-8B shape's decode at batch 1 / 8 / 64, its
-prefill and the same two further lengths, and the Qwen3-32B shape's continuous batching of 64
-requests with 2,048-token prompts under a 512-token step budget, decode-only and mixed steps timed
-apart, each with its share of the roofline), ``measured_peaks`` (what this box gives a streaming read
+32,768 tokens and a prompt of 8,192 tokens in one step, the Qwen3-8B shape's decode at batch 1 / 8 / 64 / 128 /
+256 and at batch 32 behind 16,384 tokens, its prefill and the same two further lengths, and the Qwen3-32B
+shape's continuous batching of 64 requests with 2,048-token prompts under a 512-token step budget,
+decode-only and mixed steps timed apart, its decode at batch 1 / 8 / 64 and its 2,048-token prefill, each
+with its share of the roofline), ``measured_peaks`` (what this box gives a streaming read
 and the engine's bfloat16 product) and ``sidecar`` (device, clocks and power while the headline point
 ran, versions, commit, the engine's effective configuration).
 
@@ -56,7 +57,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--warmup-seconds", type=float, default=0.3,
                     help="after the warm-up steps, repeat the last of them for at least this long and until the clock is steady")
-    ap.add_argument("--warmup-most-seconds", type=float, default=3.0, help="give up waiting for a steady clock after this long")
+    ap.add_argument("--warmup-most-seconds", type=float, default=4.5,
+                    help="give up waiting for a steady clock after this long (the firmware reports about once a second)")
     ap.add_argument("--preset", default="0.6B")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the preset has (reported in config)")
     ap.add_argument("--batch", type=int, default=8)
@@ -101,7 +103,9 @@ def main() -> int:
 
     def decode_run(model, cfg, batch, steps, warmup, describe=False, context=None):
         """Decode ``steps`` timed tokens for ``batch`` requests ending at the context length, after the
-        warm-up; returns a dict with the rate, the step time and the step's share of the roofline."""
+        warm-up; returns a dict with the rate, the step time and the step's share of the roofline. With
+        ``describe`` (the headline point) the warm-up waits for a steady clock, and the last step is kept
+        running after the timed ones until the firmware has reported on the device once more."""
         context = context or args.context
         warm_steps = max(warmup, 1)
         total = warm_steps + steps
@@ -134,9 +138,10 @@ def main() -> int:
                 eng.runner.repeat_last_step()
             torch.cuda.synchronize()
 
-        held = monitor.warm_until_steady(hold, args.warmup_seconds, max(args.warmup_seconds, args.warmup_most_seconds))
+        most = max(args.warmup_seconds, args.warmup_most_seconds) if describe else args.warmup_seconds
+        held = monitor.warm_until_steady(hold, args.warmup_seconds, most)
         warm_s = time.perf_counter() - w0
-        monitor.interval_s = 0.1  # fewer readings while the host is being timed
+        monitor.interval_s = 0.25  # fewer readings while the host is being timed
         ctx0 = sum(r.seq_len for r in reqs) / batch
         t_mark = monitor.read_now()
         with measured_region(f"decode b{batch}"):
@@ -150,8 +155,11 @@ def main() -> int:
         step_bytes = model.decode_read_bytes() + batch * mean_ctx * eng.runner.pool.bytes_per_token()
         out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "mean_ctx": mean_ctx,
                "achieved_gbs": step_bytes / (dt / steps) / 1e9, "warmup_steps": warm_steps, "warmup_s": round(warm_s, 3),
-               "held": held, "since": t_mark, "until": monitor.read_now()}
-        monitor.interval_s = 0.02
+               "held": held, "since": t_mark}
+        monitor.interval_s = 0.05
+        if describe:  # the timed steps are over in a few hundredths of a second: no refresh falls inside them
+            monitor.hold_until_refresh(hold)
+        out["until"] = monitor.read_now()
         if describe:
             out["sidecar"] = sidecar(eng)
         for r in reqs:
@@ -218,15 +226,17 @@ def main() -> int:
     cfg, full_layers, model = make(args.preset, args.layers)
     vocab = cfg["vocab_size"]
     side = {}
-    monitor = GpuMonitor().start()  # readings every 20 ms from here to the end of the run
+    monitor = GpuMonitor().start()  # polls from here to the end of the run
     if args.prefill_only:
         head = {"tok_s": 0.0, "ms_per_step": 0.0, "achieved_gbs": 0.0, "mean_ctx": 0.0, "warmup_steps": 0}
     else:
         head = decode_run(model, cfg, args.batch, args.steps, args.warmup, describe=True)
         side = head.pop("sidecar")
         side["warmup"] = {"steps": head["warmup_steps"], "seconds": head["warmup_s"], "repeats_of_the_last_step": 8 * head["held"]["calls"],
-                          "held_seconds": head["held"]["seconds"], "clock_steady": head["held"]["steady"]}
-        side["gpu_during_timed_steps"] = monitor.window(head["since"], head["until"])
+                          "held_seconds": head["held"]["seconds"], "refreshes_seen": head["held"]["refreshes"],
+                          "clock_steady": head["held"]["steady"]}
+        # the firmware's first report after the timed steps, taken while their last step was kept running
+        side["gpu_at_timed_steps"] = monitor.window(head["since"], head["until"])
     achieved = head["achieved_gbs"]
 
     out = {
@@ -315,6 +325,12 @@ def main() -> int:
         p8 = prefill_run(m8, cfg8, 8192, 0, repeats=3)
         points["8B_prefill_8192"] = p8["value"]
         points["8B_prefill_8192_frac"] = p8["frac"]
+        # larger batches, and a batch behind 16,384 tokens
+        for b, steps, ctx in ((128, 12, 4096), (256, 8, 4096), (32, 12, 16384)):
+            r = decode_run(m8, cfg8, b, steps, 4, context=ctx)
+            name = f"8B_decode_b{b}" + ("" if ctx == 4096 else f"_ctx{ctx}")
+            points[name] = round(r["tok_s"], 1)
+            points[name + "_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
         del m8
         gc.collect()
         torch.cuda.empty_cache()
@@ -322,6 +338,13 @@ def main() -> int:
         c = continuous_run(m32, cfg32)
         for k, v in c.items():
             points[f"32B_cont64_{k}"] = round(v, 4 if "frac" in k else 2)
+        for b, steps in ((1, 12), (8, 12), (64, 8)):
+            r = decode_run(m32, cfg32, b, steps, 4)
+            points[f"32B_decode_b{b}"] = round(r["tok_s"], 1)
+            points[f"32B_decode_b{b}_frac"] = round(r["achieved_gbs"] / HBM_PEAK_GBS, 4)
+        p32 = prefill_run(m32, cfg32, 2048, 0, repeats=3)
+        points["32B_prefill_2048"] = p32["value"]
+        points["32B_prefill_2048_frac"] = p32["frac"]
         del m32
         gc.collect()
         torch.cuda.empty_cache()

@@ -5,9 +5,16 @@ record beside every row of its results and warms up until the clock has settled
 library (``amdsmi``, one metrics call of a third of a millisecond per reading); readings are rows of one
 numpy array, unknown values are NaN and are reported as None, never as a guess.
 
+The firmware refreshes the figures it hands out about once a second (measured: every source of the
+library shows the same values for a second, then the next), and stamps each refresh with its own clock.
+Polling faster finds a refresh sooner but learns nothing more, so everything below counts *refreshes*:
+the first reading of each firmware time stamp. A statement about the clock therefore takes seconds, not
+tenths: the first refresh after a load begins still mixes idle and load, the two after it can agree.
+
 ``GpuMonitor`` keeps a ring of readings filled by a background thread. ``window(since, until)`` condenses
-the readings of a time span; ``steady()`` says whether the shader clock has stopped moving;
-``warm_until_steady(work, least_s, most_s)`` runs ``work()`` again and again until it has.
+the refreshes of a time span; ``steady()`` says whether the shader clock has stopped moving;
+``warm_until_steady(work, least_s, most_s)`` runs ``work()`` again and again until it has;
+``hold_until_refresh(work, most_s)`` keeps the load up until the firmware has reported on it once more.
 """
 
 from __future__ import annotations
@@ -18,9 +25,11 @@ import time
 import numpy as np
 
 # One reading: monotonic time, shader and memory clock (MHz), socket power (W), hot-spot and memory
-# temperature (C), shader and memory-controller activity (%).
-COLUMNS = ("t", "sclk_mhz", "mclk_mhz", "power_w", "temp_c", "mem_temp_c", "busy_pct", "mem_busy_pct")
-_METRIC_KEYS = {"sclk_mhz": "current_gfxclk", "mclk_mhz": "current_uclk", "power_w": "current_socket_power",
+# temperature (C), shader and memory-controller activity (%), and the firmware's time stamp of the refresh
+# the figures come from (its own units; only equality is used).
+COLUMNS = ("t", "sclk_mhz", "mclk_mhz", "power_w", "temp_c", "mem_temp_c", "busy_pct", "mem_busy_pct", "refresh")
+REPORTED = COLUMNS[1:-1]  # what summaries name
+_METRIC_KEYS = {"refresh": "firmware_timestamp", "sclk_mhz": "current_gfxclk", "mclk_mhz": "current_uclk", "power_w": "current_socket_power",
                 "temp_c": "temperature_hotspot", "mem_temp_c": "temperature_mem", "busy_pct": "average_gfx_activity",
                 "mem_busy_pct": "average_umc_activity"}
 _NAN = float("nan")
@@ -111,7 +120,7 @@ class GpuMonitor:
     """Readings of one GPU in a ring of ``capacity`` rows, taken every ``interval_s`` seconds by a thread
     between ``start()`` and ``stop()`` (or inside a ``with`` block), and on demand by ``read_now()``."""
 
-    def __init__(self, device: int = 0, interval_s: float = 0.02, capacity: int = 1 << 16):
+    def __init__(self, device: int = 0, interval_s: float = 0.05, capacity: int = 1 << 16):
         self.interval_s = interval_s
         self._dev = _Device(device)
         self._rows = np.full((capacity, len(COLUMNS)), np.nan)
@@ -175,53 +184,75 @@ class GpuMonitor:
             rows = self._rows[:n].copy() if n <= cap else np.roll(self._rows, -(n % cap), axis=0).copy()
         return rows[np.argsort(rows[:, 0], kind="stable")]
 
+    def refreshes(self, since: float | None = None, until: float | None = None) -> np.ndarray:
+        """The first reading of every refresh of the firmware's figures within the span (every reading,
+        where the firmware's time stamp is unknown)."""
+        rows = self.readings()
+        stamp = rows[:, COLUMNS.index("refresh")]
+        if len(rows) and not np.isnan(stamp).all():
+            rows = rows[np.concatenate(([True], stamp[1:] != stamp[:-1])) & ~np.isnan(stamp)]
+        t = rows[:, 0]
+        return rows[(t >= (-np.inf if since is None else since)) & (t <= (np.inf if until is None else until))]
+
     def column(self, name: str) -> np.ndarray:
         return self.readings()[:, COLUMNS.index(name)]
 
     def window(self, since: float | None = None, until: float | None = None) -> dict:
-        """Count, and per column lowest, highest and mean of the known readings, of the span."""
-        rows = self.readings()
-        t = rows[:, 0]
-        rows = rows[(t >= (-np.inf if since is None else since)) & (t <= (np.inf if until is None else until))]
+        """Count of refreshes, and per figure lowest, highest and mean of the known ones, of the span."""
+        rows = self.refreshes(since, until)
         out = {"samples": int(len(rows))}
-        for i, col in enumerate(COLUMNS[1:], 1):
-            known = rows[:, i][~np.isnan(rows[:, i])]
+        for col in REPORTED:
+            v = rows[:, COLUMNS.index(col)]
+            known = v[~np.isnan(v)]
             out[col] = None if known.size == 0 else {"min": float(known.min()), "max": float(known.max()),
                                                      "mean": round(float(known.mean()), 1)}
         return out
 
-    def steady(self, readings: int = 5, tolerance: float = 0.02) -> bool | None:
-        """Whether the shader clock has stopped moving: the mean of its latest ``readings`` known values lies
-        within ``tolerance`` of the mean of the ``readings`` before them (the reference's rule,
-        bench/sidecar.py:187-196). None while fewer than twice ``readings`` are known."""
-        clock = self.column("sclk_mhz")
+    @staticmethod
+    def _agree(clock: np.ndarray, readings: int, tolerance: float) -> bool | None:
         clock = clock[~np.isnan(clock)]
         if clock.size < 2 * readings:
             return None
         latest, earlier = clock[-readings:].mean(), clock[-2 * readings : -readings].mean()
         return bool(latest > 0 and abs(latest - earlier) <= tolerance * latest)
 
-    def warm_until_steady(self, work, least_s: float, most_s: float, readings: int = 5, tolerance: float = 0.02) -> dict:
+    def steady(self, readings: int = 1, tolerance: float = 0.02, since: float | None = None) -> bool | None:
+        """Whether the shader clock has stopped moving: the mean of its latest ``readings`` refreshes lies
+        within ``tolerance`` of the mean of the ``readings`` before them (the reference's rule,
+        bench/sidecar.py:187-196, over refreshes instead of samples). None while fewer than twice
+        ``readings`` are known."""
+        return self._agree(self.refreshes(since)[:, COLUMNS.index("sclk_mhz")], readings, tolerance)
+
+    def warm_until_steady(self, work, least_s: float, most_s: float, readings: int = 1, tolerance: float = 0.02) -> dict:
         """Call ``work()`` (which must leave the device busy and return when its work is done) until at
-        least ``least_s`` have passed and the clock is steady, or ``most_s`` have passed. Only readings
-        taken since the call began count. Returns what happened: calls, seconds, and ``steady`` (None when
-        the clock could not be read often enough to tell)."""
+        least ``least_s`` have passed and the clock is steady, or ``most_s`` have passed. Of the refreshes
+        since the call began the first does not count: it mixes what came before with the load. Returns
+        what happened: calls, seconds, refreshes seen, and ``steady`` (None when the clock could not be read
+        often enough to tell)."""
         began = time.monotonic()
-        calls, verdict = 0, None
+        calls, verdict, seen = 0, None, 0
         while True:
             work()
             calls += 1
             spent = time.monotonic() - began
             if spent < least_s:
                 continue
-            clock = self.readings()
-            clock = clock[clock[:, 0] >= began][:, COLUMNS.index("sclk_mhz")]
-            clock = clock[~np.isnan(clock)]
-            if clock.size >= 2 * readings:
-                latest, earlier = clock[-readings:].mean(), clock[-2 * readings : -readings].mean()
-                verdict = bool(latest > 0 and abs(latest - earlier) <= tolerance * latest)
+            clock = self.refreshes(began)[1:, COLUMNS.index("sclk_mhz")]
+            seen = int(clock.size)
+            verdict = self._agree(clock, readings, tolerance)
             if verdict or spent >= most_s:
-                return {"calls": calls, "seconds": round(spent, 3), "steady": verdict}
+                return {"calls": calls, "seconds": round(spent, 3), "refreshes": seen, "steady": verdict}
+
+    def hold_until_refresh(self, work, most_s: float = 1.5) -> bool:
+        """Call ``work()`` until the firmware has refreshed its figures once more (so that a span too short
+        to hold a refresh is followed by one taken under the same load), or ``most_s`` have passed."""
+        began = time.monotonic()
+        before = len(self.refreshes())
+        while time.monotonic() - began < most_s:
+            work()
+            if len(self.refreshes()) > before:
+                return True
+        return False
 
     def conditions(self) -> dict:
         """What the run was bounded by: limits, and the share of time the firmware held the device back
@@ -234,7 +265,7 @@ class GpuMonitor:
 def gpu_now(device: int = 0) -> dict:
     """One reading as a dictionary (None = unknown), without its time."""
     row = _Device(device).read()
-    return {c: (None if v != v else v) for c, v in zip(COLUMNS[1:], row[1:])}
+    return {c: (None if v != v else v) for c, v in zip(COLUMNS, row) if c in REPORTED}
 
 
 def sidecar(engine=None) -> dict:

@@ -48,7 +48,7 @@ def test_bench_line_on_a_tiny_shape():
     """The benchmark's one JSON line with a tiny preset: every key of the contract, the flat config of
     at most 20 keys, the prefill and roofline records, the batch 1 and 64 points, the sidecar."""
     p = run(ROOT / "bench.py", "--preset", "tinyE", "--batch", "2", "--context", "512", "--steps", "4", "--warmup", "2",
-            "--prefill-tokens", "128", "--warmup-seconds", "0.02")
+            "--prefill-tokens", "128", "--warmup-seconds", "0.02", "--warmup-most-seconds", "0.05")
     assert p.returncode == 0, p.stderr[-2000:]
     line = json.loads(p.stdout.strip().splitlines()[-1])
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
@@ -94,11 +94,11 @@ def test_the_monitor_reads_a_loaded_gpu():
 
     with GpuMonitor(interval_s=0.02) as g:
         t0 = time.monotonic()
-        out = g.warm_until_steady(work, least_s=1.0, most_s=4.0)
-        busy = g.window(since=t0 + 0.5)
+        out = g.warm_until_steady(work, least_s=1.0, most_s=5.0)
+        busy = g.window(since=t0 + 1.2)  # the first refresh after the load began may still mix idle and load
         limits = g.conditions()
     assert out["steady"] is not None, "the clock could be read often enough to decide"
-    assert busy["samples"] >= 10
+    assert busy["samples"] >= 2, "the firmware refreshes its figures about once a second"
     assert busy["sclk_mhz"]["mean"] > 1000, busy
     assert 50 < busy["power_w"]["mean"] < 2000 and busy["power_w"]["max"] < 2000, busy
     assert busy["mclk_mhz"]["mean"] > 500 and 10 < busy["temp_c"]["mean"] < 120, busy

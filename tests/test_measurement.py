@@ -17,9 +17,11 @@ from miniserve_amd.measurement.offline import run_to_completion
 from miniserve_amd.measurement.sidecar import COLUMNS, throttled_share
 
 
-def readings(clocks, power=None, t0=100.0, dt=0.1):
-    """Rows in the monitor's column order: time, shader clock, memory clock, power, two temperatures, two activities."""
-    return [(t0 + i * dt, c, 2000.0, None if power is None else power[i], 40.0, 35.0, 99.0, 10.0) for i, c in enumerate(clocks)]
+def readings(clocks, power=None, t0=100.0, dt=0.1, polls=1):
+    """Rows in the monitor's column order: time, shader clock, memory clock, power, two temperatures, two
+    activities, the firmware's stamp of the refresh. Every refresh is read ``polls`` times in a row."""
+    return [(t0 + (i * polls + k) * dt / polls, c, 2000.0, None if power is None else power[i], 40.0, 35.0, 99.0, 10.0, 7000 + i)
+            for i, c in enumerate(clocks) for k in range(polls)]
 
 
 def monitor_with(rows, **kw):
@@ -30,7 +32,7 @@ def monitor_with(rows, **kw):
 
 def test_a_reading_without_a_gpu_says_unknown_not_zero():
     s = gpu_now()
-    assert set(s) == set(COLUMNS[1:]) and "power_w" in s and "mclk_mhz" in s
+    assert set(s) == set(COLUMNS[1:-1]) and "power_w" in s and "mclk_mhz" in s and "refresh" not in s
     assert all(v is None or v >= 0 for v in s.values())
 
 
@@ -45,6 +47,12 @@ def test_the_clock_is_steady_when_two_runs_of_readings_agree():
     assert monitor_with(readings([None] * 20)).steady() is None, "a clock that cannot be read settles nothing"
     gaps = monitor_with(readings([1700, None, 1700, 1700, None, 1700, 1700, 1700, 1700, 1700]))  # unknown readings are skipped
     assert gaps.steady(readings=4) is True
+    # what counts are the firmware's refreshes, however often each is read: two refreshes polled ten times each decide
+    # what two refreshes decide, not what twenty readings would
+    polled = monitor_with(readings([2400, 2300, 1700, 1700], polls=10))
+    assert len(polled.readings()) == 40 and len(polled.refreshes()) == 4
+    assert polled.steady(readings=1) is True and polled.steady(readings=2) is False and polled.steady(readings=4) is None
+    assert polled.window()["samples"] == 4 and polled.window()["sclk_mhz"]["mean"] == 2025.0
 
 
 def test_the_window_covers_the_timed_span_only():
@@ -55,7 +63,7 @@ def test_the_window_covers_the_timed_span_only():
     assert inside["samples"] == 3 and inside["sclk_mhz"] == {"min": 1700, "max": 1800, "mean": 1733.3}
     assert inside["power_w"] == {"min": 900, "max": 1000, "mean": 966.7} and inside["mclk_mhz"]["mean"] == 2000.0
     empty = g.window(since=200.0)
-    assert empty["samples"] == 0 and all(empty[c] is None for c in COLUMNS[1:])
+    assert empty["samples"] == 0 and all(empty[c] is None for c in COLUMNS[1:-1])
     g = monitor_with(readings([None, None]))
     assert g.window()["sclk_mhz"] is None and g.window()["temp_c"]["mean"] == 40.0
 
@@ -82,23 +90,43 @@ def test_warming_waits_for_a_steady_clock_between_a_least_and_a_most_time():
     """``work`` stands for a few decode steps; the readings are fed by the test instead of a thread."""
     g = GpuMonitor()
     clocks = iter([2400, 2300, 2200, 2100, 2000, 1900, 1800] + [1700] * 200)
+    stamp = iter(range(10**6))
 
     def work():
-        g._append([time.monotonic(), next(clocks), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0])
+        g._append([time.monotonic(), next(clocks), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0, next(stamp)])
         time.sleep(0.004)
 
     out = g.warm_until_steady(work, least_s=0.02, most_s=2.0, readings=3)
-    # falling for seven readings, then flat: steady once the last three and the three before them agree
-    assert out["steady"] is True and 0.02 <= out["seconds"] < 1.0 and 10 <= out["calls"] < 100
+    # falling for seven refreshes, then flat: steady once the last three and the three before them agree
+    assert out["steady"] is True and 0.02 <= out["seconds"] < 1.0 and 10 <= out["calls"] < 100 and out["refreshes"] >= 6
     falling = iter(range(2400, 0, -20))
     g2 = GpuMonitor()
 
     def cooling():
-        g2._append([time.monotonic(), next(falling), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0])
+        g2._append([time.monotonic(), next(falling), 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0, next(stamp)])
         time.sleep(0.004)
 
     out = g2.warm_until_steady(cooling, least_s=0.01, most_s=0.15, readings=3)
     assert out["steady"] is False and out["seconds"] >= 0.15, "a clock that keeps moving ends the wait at the most time, and says so"
+    # the first refresh after the warm-up began mixes what came before with the load and does not count:
+    # idle, then the load's clock twice, is steady at the third refresh and not at the second
+    g4 = GpuMonitor()
+    seen = iter([(900, 1), (900, 1), (2000, 2), (2000, 2), (2000, 3)] + [(2000, 3)] * 100)
+
+    def slow_firmware():
+        c, s = next(seen)
+        g4._append([time.monotonic(), c, 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0, 5000 + s])
+        time.sleep(0.004)
+
+    out = g4.warm_until_steady(slow_firmware, least_s=0.0, most_s=1.0)
+    assert out == {"calls": 5, "seconds": out["seconds"], "refreshes": 2, "steady": True}
+    # and a load kept up until the firmware reports once more
+    g5 = GpuMonitor()
+    ticks = iter([4, 4, 4, 5, 5])
+    g5._append([time.monotonic(), 2000, 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0, 4])
+    assert g5.hold_until_refresh(lambda: g5._append([time.monotonic(), 2000, 2000.0, 900.0, 50.0, 40.0, 100.0, 20.0, next(ticks)])) is True
+    assert len(g5.refreshes()) == 2 and len(g5.readings()) == 5
+    assert g5.hold_until_refresh(lambda: time.sleep(0.01), most_s=0.03) is False
     g3 = GpuMonitor()
     out = g3.warm_until_steady(lambda: time.sleep(0.002), least_s=0.01, most_s=0.03)
     assert out["steady"] is None and out["seconds"] >= 0.03, "a clock that cannot be read decides nothing"
