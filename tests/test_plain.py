@@ -137,6 +137,35 @@ def test_swiglu():
     assert not np.allclose(P.swiglu(x, wg, wu, wd), P.swiglu(x, wu, wg, wd))  # gate and up are not interchangeable
 
 
+def test_the_reference_says_both_formulas_twice():
+    """The direction of the turn and which of gate / up goes through SiLU are stated twice in the reference, in
+    different words: once as written-out arithmetic (model/qwen3.py:85-87,107-108,128-131, what ``tests/plain``
+    follows) and once as calls of library operators in its fused path, whose published meanings are fixed
+    outside the reference: ``apply_rope_with_cos_sin_cache_inplace(..., is_neox=True)`` over a table of one
+    row ``[cos(angles), sin(angles)]`` per token (model/fused.py:182-184,209: the halves of a head are the
+    pairs, ``first' = first cos - second sin``, ``second' = second cos + first sin``), and ``silu_and_mul``
+    over the product with the concatenated weight, gate rows first (model/fused.py:41,195:
+    ``silu(y[..., :I]) * y[..., I:]``). The reference's own tests hold the two paths equal on a real checkpoint
+    (tests/test_fused.py:71-141). Written here from the second statement and compared with the first."""
+    d, t = 16, 5
+    x = rng.standard_normal((t, 3, d))
+    pos = np.array([0, 1, 7, 300, 4000])
+    ang = P.rotary_angles(pos, d, 1e6).astype(np.float64)
+    table = np.concatenate((np.cos(ang), np.sin(ang)), axis=-1)  # one row per token: cosines, then sines
+    cos, sin = table[:, None, : d // 2], table[:, None, d // 2 :]
+    first, second = x[..., : d // 2], x[..., d // 2 :]
+    neox = np.concatenate((first * cos - second * sin, second * cos + first * sin), axis=-1)
+    assert np.allclose(P.apply_rotary(x, ang.astype(np.float32)), neox, atol=1e-12)
+    other_way = np.concatenate((first * cos + second * sin, second * cos - first * sin), axis=-1)
+    assert not np.allclose(neox, other_way)
+    h, inter = 6, 10
+    y = rng.standard_normal((4, h))
+    wg, wu, wd = rng.standard_normal((inter, h)), rng.standard_normal((inter, h)), rng.standard_normal((h, inter))
+    both = y @ np.concatenate((wg, wu), axis=0).T  # gate rows first
+    silu_and_mul = both[:, :inter] / (1 + np.exp(-both[:, :inter])) * both[:, inter:]
+    assert np.allclose(P.swiglu(y, wg, wu, wd), silu_and_mul @ wd.T)
+
+
 # ------------------------------------------------------------------------------------------ the whole model
 
 
