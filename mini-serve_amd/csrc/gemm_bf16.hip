@@ -4,6 +4,9 @@
 //  * tile kernel, slabs straight into LDS (prefill, M large, K a multiple of 64): 128 x 128 macro-tiles,
 //                  K-slabs of 64 loaded by global_load_lds into a ring of two stages with a bank
 //                  swizzle, one barrier per slab, two blocks per CU; 4 waves in a 2 x 2 grid of wave tiles.
+//                  Its largest form, 256 x 256 with four wave tiles of 128 x 128, has its loop over K
+//                  written in assembly (all 512 registers of a lane, fragment reads and loads placed
+//                  between the products by hand) and one block per CU that takes tiles in turn.
 //  * tile kernel, slabs through registers (any K and alignment, or few tiles): BM x BN macro-tiles
 //                  staged through LDS in K-slabs of 64 with a register prefetch of the next slab.
 //  * small-M kernel (decode, M <= 64): pure weight streaming. A wave owns 16 weight rows and a slice
@@ -19,6 +22,8 @@
 // Any permutation of k that is the same for both operands leaves the result unchanged; the small-M
 // kernel uses that to let a lane load 16 consecutive k at once.
 #include "common.h"
+
+#include <utility>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -67,6 +72,18 @@ __device__ __forceinline__ void store4(void* __restrict__ C, int mode, int m, in
       else ((float*)C)[at + i] += a[i];
     }
   }
+}
+
+// SiLU and tanh-GELU on the hardware's exp2 and reciprocal (about 1 ulp each, in float32): what they lose
+// disappears in the rounding to bfloat16, and the library forms take some 35 instructions a value, which in
+// the epilogue of the gated tile product was a tenth of the kernel's time.
+__device__ __forceinline__ float activate_fast(float x, int act) {
+  if (act == MS_ACT_GELU_TANH) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    const float t = 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(u * 2.885390081777927f));  // tanh(u)
+    return 0.5f * x * (1.f + t);
+  }
+  return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -213,9 +230,9 @@ __device__ __forceinline__ void banded(int t, int rows, int cols, int band_cols,
 // caller has checked that the tile counts divide) the XCDs form a grid of xcd_rows x 8 / xcd_rows, each
 // owning a rectangle of tiles that it walks in banded order: then an XCD reads only its share of the
 // activations, which is what counts when the weight matrix is the smaller operand.
-__device__ __forceinline__ TileId tile_of_block(int block, int row_tiles, int col_tiles, int xcd_rows, int band_cols) {
+__device__ __forceinline__ TileId tile_of_block(int block, int blocks, int row_tiles, int col_tiles, int xcd_rows, int band_cols) {
   const int tiles = row_tiles * col_tiles;
-  const int splits = gridDim.x / tiles;
+  const int splits = blocks / tiles;
   TileId id;
   int t;
   if (row_tiles == 1 && splits > 1) {
@@ -260,7 +277,7 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
 
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 16, g = lane / 16;
-  const TileId id = tile_of_block(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, xcd_rows, band_cols);
+  const TileId id = tile_of_block(blockIdx.x, gridDim.x, (M + BM - 1) / BM, (N + BN - 1) / BN, xcd_rows, band_cols);
   const int m0 = id.m * BM, n0 = id.n * BN;
   const int wm = (wave / WC) * WM, wn = (wave % WC) * WN;
   const int k_lo = id.split * k_per;
@@ -368,6 +385,384 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
 #pragma unroll
     for (int j = 0; j < FM; ++j)
       store4(C, mode, m0 + wm + j * 16 + r, n0 + wn + i * 16 + g * 4, M, N, ldc, acc[i][j], vec_store);
+}
+
+// ---------------------------------------------------------------------------------------------
+// 256 x 256 tile with four waves, each with a wave tile of 128 x 128: 16 fragment reads for 64
+// products (the eight-wave tile above reads 12 for 32), so that fragment reads and the loads into LDS
+// together keep the LDS busy three quarters of the time the products take instead of all of it. The 256
+// accumulator registers of a lane are all the AGPRs there are, and one wave per SIMD has nobody to
+// cover its waits, so registers and instruction order of the loop over K are written out: the loop is
+// one assembly statement. Layout of LDS, swizzle and operand roles are those of the kernel above.
+//   registers: a[4 (8 i + j) ..] accumulators of fragment (i = weight block, j = row block)
+//              v[128 + 4 i ..], v[160 + 4 j ..]  fragment set A (even 32-k steps: weights, rows)
+//              v[192 + 4 i ..], v[224 + 4 j ..]  fragment set B (odd steps)
+//              v[96 .. 111] byte offsets of this lane's 16 loads of a slab (8 of rows, 8 of weights)
+//              v[112 .. 115] LDS addresses of the fragment reads (weights step 0 / 1, rows step 0 / 1)
+//              s[80:81], s[82:83] where the next slab to load begins (rows, weights); s84 LDS address of
+//              this wave's part of the stage it loads into; s85 distance to the other stage (its sign
+//              alternates); s86 slabs left
+//   per slab:  step 0: products on set A, between them the reads of set B (same slab, second step);
+//              wait for the next slab's loads, barrier (every wave has read all it needs of this slab);
+//              step 1: products on set B, between them the reads of set A from the next slab and the
+//              loads of the slab after next into this slab's stage.
+// The slab count must be at least 2 (the caller checks); rows beyond M or N read the last valid row.
+// Between the assembly statement and the reads of the accumulators after it the compiler must leave the
+// AGPRs alone: it has no use for them here (no matrix builtins, 96 VGPRs of its own and nothing spilled:
+// the kernel's scratch size is 0), and every statement names all of them as clobbered.
+// One block per CU stays for the whole product and takes tiles in turn. Measured at 8192^3, sustained, at
+// the socket's power limit: 1,500 TFLOP/s against 1,260 of the eight-wave tile and 1,620 of the vendor
+// library; at 2,048 x 24,576 x 4,096 1,506 against 1,175 and 1,530.
+
+// Accumulator fragment F of the wide tile's loop, out of the AGPRs.
+template <int F>
+__device__ __forceinline__ floatx4 wide_acc() {
+  floatx4 v;
+  asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%4+1]\n\tv_accvgpr_read_b32 %2, a[%4+2]\n\tv_accvgpr_read_b32 %3, a[%4+3]"
+               : "=v"(v[0]), "=v"(v[1]), "=v"(v[2]), "=v"(v[3])
+               : "n"(F * 4));
+  return v;
+}
+
+// Four consecutive n of row m: the store of one accumulator fragment. MODE 0: bf16, 1: float, 2: float +=.
+// INSIDE: the tile lies wholly within the matrix and rows are 8-byte aligned, so nothing is tested.
+template <int MODE, bool INSIDE>
+__device__ __forceinline__ void store_fragment(void* __restrict__ C, int m, int n, int M, int N, int ldc, floatx4 a, bool vec_ok) {
+  if constexpr (!INSIDE) {
+    store4(C, MODE, m, n, M, N, ldc, a, vec_ok);
+  } else {
+    const size_t at = (size_t)m * ldc + n;
+    if constexpr (MODE == 0) {
+      union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.e[i] = static_cast<bf16>(a[i]);
+      *reinterpret_cast<uint2*>((bf16*)C + at) = o.u;
+    } else if constexpr (MODE == 1) {
+      *reinterpret_cast<float4*>((float*)C + at) = make_float4(a[0], a[1], a[2], a[3]);
+    } else {
+      float4 c = *reinterpret_cast<float4*>((float*)C + at);
+      c.x += a[0]; c.y += a[1]; c.z += a[2]; c.w += a[3];
+      *reinterpret_cast<float4*>((float*)C + at) = c;
+    }
+  }
+}
+
+// Gate and up fragments of the same four outputs (W holds alternating blocks of 16 gate rows and 16 up
+// rows): out[m, col ..] = act(gate) * up, bf16 with row stride ldc; `half` = N / 2 columns.
+template <int ACT, bool INSIDE>
+__device__ __forceinline__ void store_gated(bf16* __restrict__ out, int m, int col, int M, int half, int ldc, floatx4 gate, floatx4 up) {
+  if (!INSIDE && (m >= M || col >= half)) return;
+  union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(activate_fast(gate[e], ACT) * up[e]);
+  *reinterpret_cast<uint2*>(out + (size_t)m * ldc + col) = o.u;
+}
+
+// Fragments (2 P, J) and (2 P + 1, J) of the wide tile. MODE 0 to 2: stored as they are; 3 + an MS_ACT_*
+// number: as gate and up. m: this lane's row in row block 0; nb: the wave tile's first column; g: the
+// lane's group of four columns.
+template <int MODE, bool INSIDE, int P, int J>
+__device__ __forceinline__ void wide_store(void* C, void* Cbase, int m, int nb, int g, int M, int N, int ldc, bool vec_store) {
+  const floatx4 a = wide_acc<(2 * P) * 8 + J>(), b = wide_acc<(2 * P + 1) * 8 + J>();
+  const int row = m + J * 16;
+  if constexpr (MODE >= 3) {
+    store_gated<MODE - 3, INSIDE>((bf16*)Cbase, row, nb / 2 + P * 16 + g * 4, M, N / 2, ldc, a, b);
+  } else {
+    store_fragment<MODE, INSIDE>(C, row, nb + (2 * P) * 16 + g * 4, M, N, ldc, a, vec_store);
+    store_fragment<MODE, INSIDE>(C, row, nb + (2 * P + 1) * 16 + g * 4, M, N, ldc, b, vec_store);
+  }
+}
+
+template <int MODE, bool INSIDE, int... I>
+__device__ __forceinline__ void wide_stores(std::integer_sequence<int, I...>, void* C, void* Cbase, int m, int nb, int g, int M, int N,
+                                            int ldc, bool vec_store) {
+  (wide_store<MODE, INSIDE, I / 8, I % 8>(C, Cbase, m, nb, g, M, N, ldc, vec_store), ...);
+}
+
+// The same through LDS, for bfloat16 outputs of tiles that lie wholly inside the matrix with 16-byte
+// aligned rows: a lane's four values of a row go into the wave's own part of LDS (rows padded by 16
+// bytes: conflict-free), then every lane takes 16 bytes of a row back, so that a store instruction
+// writes whole 128-byte lines (four rows' worth) instead of 32-byte pieces of sixteen rows. The pieces
+// cost four times the requests at the L2, and a tile's stores then took as long as ten slabs of products.
+constexpr int WIDE_STAGED_BYTES = 128 * (256 + 16);  // per wave: 128 rows of 128 bf16
+template <int MODE, int P, int J>
+__device__ __forceinline__ void wide_stage(unsigned char* part, int r, int g) {
+  const floatx4 a = wide_acc<(2 * P) * 8 + J>(), b = wide_acc<(2 * P + 1) * 8 + J>();
+  constexpr int STRIDE = (MODE >= 3 ? 128 : 256) + 16;
+  unsigned char* row = part + (J * 16 + r) * STRIDE;
+  union { uint2 u; bf16 e[4]; } o;
+  if constexpr (MODE >= 3) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(activate_fast(a[e], MODE - 3) * b[e]);
+    *reinterpret_cast<uint2*>(row + (P * 16 + g * 4) * 2) = o.u;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(a[e]);
+    *reinterpret_cast<uint2*>(row + ((2 * P) * 16 + g * 4) * 2) = o.u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(b[e]);
+    *reinterpret_cast<uint2*>(row + ((2 * P + 1) * 16 + g * 4) * 2) = o.u;
+  }
+}
+template <int MODE, int... I>
+__device__ __forceinline__ void wide_stage_all(std::integer_sequence<int, I...>, unsigned char* part, int r, int g) {
+  (wide_stage<MODE, I / 8, I % 8>(part, r, g), ...);
+}
+// out: the wave tile's first output element; MODE 0 or 3 + an MS_ACT_* number.
+template <int MODE>
+__device__ __forceinline__ void wide_store_staged(bf16* __restrict__ out, int ldc, unsigned char* part, int lane) {
+  wide_stage_all<MODE>(std::make_integer_sequence<int, 32>{}, part, lane % 16, lane / 16);
+  constexpr int CHUNKS = MODE >= 3 ? 8 : 16, STRIDE = CHUNKS * 16 + 16, ROWS = 64 / CHUNKS;
+  const int lrow = lane / CHUNKS, ch = lane % CHUNKS;
+#pragma unroll 8
+  for (int it = 0; it < 128 / ROWS; ++it) {
+    const int row = it * ROWS + lrow;
+    const uint4 v = *reinterpret_cast<const uint4*>(part + row * STRIDE + ch * 16);
+    *reinterpret_cast<uint4*>(out + (size_t)row * ldc + ch * 8) = v;
+  }
+}
+
+// The mode is told apart once, not per fragment: each mode's stores are one straight run of code.
+template <bool INSIDE>
+__device__ __forceinline__ void wide_epilogue(void* C, void* Cbase, int mode, int m, int nb, int g, int M, int N, int ldc, bool vec_store) {
+  constexpr auto all = std::make_integer_sequence<int, 32>{};
+  static_assert(MS_ACT_COUNT == 2, "one case per activation below");
+  switch (mode) {
+    case 0: wide_stores<0, INSIDE>(all, C, Cbase, m, nb, g, M, N, ldc, vec_store); break;
+    case 1: wide_stores<1, INSIDE>(all, C, Cbase, m, nb, g, M, N, ldc, vec_store); break;
+    case 2: wide_stores<2, INSIDE>(all, C, Cbase, m, nb, g, M, N, ldc, vec_store); break;
+    case 3: wide_stores<3, INSIDE>(all, C, Cbase, m, nb, g, M, N, ldc, vec_store); break;
+    default: wide_stores<4, INSIDE>(all, C, Cbase, m, nb, g, M, N, ldc, vec_store); break;
+  }
+}
+
+// Names of registers 96 to 255 (VGPRs) and 0 to 255 (AGPRs) for the loop's clobber list.
+#define MS_R10(p, t) p #t "0", p #t "1", p #t "2", p #t "3", p #t "4", p #t "5", p #t "6", p #t "7", p #t "8", p #t "9"
+#define MS_R100_249(p)                                                                                                  \
+  MS_R10(p, 10), MS_R10(p, 11), MS_R10(p, 12), MS_R10(p, 13), MS_R10(p, 14), MS_R10(p, 15), MS_R10(p, 16), MS_R10(p, 17), \
+      MS_R10(p, 18), MS_R10(p, 19), MS_R10(p, 20), MS_R10(p, 21), MS_R10(p, 22), MS_R10(p, 23), MS_R10(p, 24)
+#define MS_R250_255(p) p "250", p "251", p "252", p "253", p "254", p "255"
+#define MS_WIDE_VGPRS "v96", "v97", "v98", "v99", MS_R100_249("v"), MS_R250_255("v")
+#define MS_WIDE_AGPRS                                                                                                   \
+  MS_R10("a", ), MS_R10("a", 1), MS_R10("a", 2), MS_R10("a", 3), MS_R10("a", 4), MS_R10("a", 5), MS_R10("a", 6),        \
+      MS_R10("a", 7), MS_R10("a", 8), MS_R10("a", 9), MS_R100_249("a"), MS_R250_255("a")
+__global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
+                                                                void* __restrict__ Cbase, int mode, int M, int N, int Kfull,
+                                                                int ldx, int ldc, int k_per, size_t c_split_stride,
+                                                                int xcd_rows, int band_cols, int items) {
+  constexpr int BM = 256, BN = 256, KS = 64, ROW_BYTES = KS * 2, STAGE_BYTES = (BM + BN) * ROW_BYTES;
+  static_assert(STAGE_BYTES == 0x10000, "the loop flips stages by 64 KB");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // 2 * STAGE_BYTES, and 4 * WIDE_STAGED_BYTES for the stores
+
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int wm = (wave / 2) * 128, wn = (wave % 2) * 128;
+  // A block works through items blockIdx.x, + gridDim.x, ...: one block per CU stays for the whole product, so
+  // that a tile's stores drain and the next tile's first loads fly while no block has to end and another
+  // to start in between. (The grid is a multiple of 8 or a single round: item L runs on XCD L % 8.)
+  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+  const TileId id = tile_of_block(item, items, (M + BM - 1) / BM, (N + BN - 1) / BN, xcd_rows, band_cols);
+  const int m0 = id.m * BM, n0 = id.n * BN;
+  const int k_lo = id.split * k_per;
+  const int K = min(Kfull, k_lo + k_per);
+  const int slabs = (K - k_lo) / KS;
+  void* C = mode == 1 ? (void*)((float*)Cbase + id.split * c_split_stride) : Cbase;
+
+  // Load side: instruction j of this wave fills tile rows (8 wave + j) * 8 .. + 7, a lane 16 bytes of one.
+  const int lrow = lane / 8, lslot = lane % 8;
+  unsigned xo[8], wo[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int R = (wave * 8 + j) * 8 + lrow;
+    const unsigned chunk = (unsigned)((lslot ^ ((R >> 1) & 7)) * 16);
+    xo[j] = (unsigned)(min(m0 + R, M - 1) - m0) * (unsigned)ldx * 2u + chunk;
+    wo[j] = (unsigned)(min(n0 + R, N - 1) - n0) * (unsigned)Kfull * 2u + chunk;
+  }
+  const unsigned long long xb = (unsigned long long)(X + (size_t)m0 * ldx + k_lo);
+  const unsigned long long wb = (unsigned long long)(W + (size_t)n0 * Kfull + k_lo);
+  // The same for every lane, which the compiler cannot tell: into scalar registers by hand.
+  const unsigned xb_lo = __builtin_amdgcn_readfirstlane((unsigned)xb), xb_hi = __builtin_amdgcn_readfirstlane((unsigned)(xb >> 32));
+  const unsigned wb_lo = __builtin_amdgcn_readfirstlane((unsigned)wb), wb_hi = __builtin_amdgcn_readfirstlane((unsigned)(wb >> 32));
+  const unsigned slabs_left = __builtin_amdgcn_readfirstlane((unsigned)slabs);
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+  const unsigned dma = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * 8192u);
+  // Read side: the rows of a fragment are base + r with base a multiple of 16, so the slot of chunk c
+  // is c ^ (r >> 1) for every fragment; step t reads chunk column 4 t + g.
+  const unsigned sw = (unsigned)(r >> 1) & 7u;
+  const unsigned raw0 = lds0 + BM * ROW_BYTES + (unsigned)(wn + r) * ROW_BYTES + (((unsigned)g ^ sw) * 16u);
+  const unsigned raw1 = lds0 + BM * ROW_BYTES + (unsigned)(wn + r) * ROW_BYTES + (((unsigned)(4 + g) ^ sw) * 16u);
+  const unsigned rax0 = lds0 + (unsigned)(wm + r) * ROW_BYTES + (((unsigned)g ^ sw) * 16u);
+  const unsigned rax1 = lds0 + (unsigned)(wm + r) * ROW_BYTES + (((unsigned)(4 + g) ^ sw) * 16u);
+
+// Between the 64 products of a step: a fragment read after every third (all 16 are out 18 products
+// before the step ends, so the next step starts without waiting for them), a load into LDS after every
+// fourth (all 16 at once, right after the barrier, measured 11 % slower: the loads' LDS writes then
+// crowd out the fragment reads).
+#define MS_WIDE_READ_EVERY 3
+#define MS_WIDE_READ_FIRST 1
+#define MS_WIDE_LOAD_EVERY 4
+#define MS_STR2(x) #x
+#define MS_STR(x) MS_STR2(x)
+  asm volatile(".set ms_read_every, " MS_STR(MS_WIDE_READ_EVERY) "\n.set ms_read_first, " MS_STR(MS_WIDE_READ_FIRST) "\n.set ms_load_every, " MS_STR(MS_WIDE_LOAD_EVERY) "\n" R"(
+    .macro MS_WIDE_MFMA mi, cw, cx
+      v_mfma_f32_16x16x32_bf16 a[(\mi)*4:(\mi)*4+3], v[\cw+((\mi)>>3)*4:\cw+((\mi)>>3)*4+3], v[\cx+((\mi)&7)*4:\cx+((\mi)&7)*4+3], a[(\mi)*4:(\mi)*4+3]
+    .endm
+    .macro MS_WIDE_READ q, nw, nx, aw, ax
+      .if (\q) < 8
+        ds_read_b128 v[\nw+(\q)*4:\nw+(\q)*4+3], v[\aw] offset:(\q)*2048
+      .else
+        ds_read_b128 v[\nx+((\q)-8)*4:\nx+((\q)-8)*4+3], v[\ax] offset:((\q)-8)*2048
+      .endif
+    .endm
+    .macro MS_WIDE_LOAD_TO q
+      s_add_u32 m0, s84, (\q)*1024+((\q)>>3)*24576
+    .endm
+    .macro MS_WIDE_LOAD q
+      .if (\q) < 8
+        global_load_lds_dwordx4 v[96+(\q)], s[80:81]
+      .else
+        global_load_lds_dwordx4 v[96+(\q)], s[82:83]
+      .endif
+    .endm
+    .macro MS_WIDE_SLAB_LOADS
+      .set ms_q, 0
+      .rept 16
+        MS_WIDE_LOAD_TO ms_q
+        s_nop 0
+        MS_WIDE_LOAD ms_q
+        .set ms_q, ms_q+1
+      .endr
+      s_add_u32 s80, s80, 128
+      s_addc_u32 s81, s81, 0
+      s_add_u32 s82, s82, 128
+      s_addc_u32 s83, s83, 0
+    .endm
+    .macro MS_WIDE_STEP cw, cx, nw, nx, aw, ax, loads
+      .set ms_mi, 0
+      .rept 64
+        .if \loads
+          .if ((ms_mi-(ms_mi/ms_load_every)*ms_load_every) == ms_load_every-1) && ((ms_mi/ms_load_every) < 16)
+            MS_WIDE_LOAD_TO (ms_mi/ms_load_every)
+          .endif
+        .endif
+        MS_WIDE_MFMA ms_mi, \cw, \cx
+        .if ((ms_mi-(ms_mi/ms_read_every)*ms_read_every) == ms_read_first) && ((ms_mi/ms_read_every) < 16)
+          MS_WIDE_READ (ms_mi/ms_read_every), \nw, \nx, \aw, \ax
+        .endif
+        .if \loads
+          .if ((ms_mi-(ms_mi/ms_load_every)*ms_load_every) == ms_load_every-1) && ((ms_mi/ms_load_every) < 16)
+            MS_WIDE_LOAD (ms_mi/ms_load_every)
+          .endif
+        .endif
+        .set ms_mi, ms_mi+1
+      .endr
+    .endm
+
+    v_mov_b32 v96, %[xo0]
+    v_mov_b32 v97, %[xo1]
+    v_mov_b32 v98, %[xo2]
+    v_mov_b32 v99, %[xo3]
+    v_mov_b32 v100, %[xo4]
+    v_mov_b32 v101, %[xo5]
+    v_mov_b32 v102, %[xo6]
+    v_mov_b32 v103, %[xo7]
+    v_mov_b32 v104, %[wo0]
+    v_mov_b32 v105, %[wo1]
+    v_mov_b32 v106, %[wo2]
+    v_mov_b32 v107, %[wo3]
+    v_mov_b32 v108, %[wo4]
+    v_mov_b32 v109, %[wo5]
+    v_mov_b32 v110, %[wo6]
+    v_mov_b32 v111, %[wo7]
+    v_mov_b32 v112, %[raw0]
+    v_mov_b32 v113, %[raw1]
+    v_mov_b32 v114, %[rax0]
+    v_mov_b32 v115, %[rax1]
+    s_mov_b32 s80, %[xb_lo]
+    s_mov_b32 s81, %[xb_hi]
+    s_mov_b32 s82, %[wb_lo]
+    s_mov_b32 s83, %[wb_hi]
+    s_mov_b32 s84, %[dma]
+    s_mov_b32 s85, 0x10000
+    s_mov_b32 s86, %[slabs]
+    .set ms_q, 0
+    .rept 256
+      v_accvgpr_write_b32 a[ms_q], 0
+      .set ms_q, ms_q+1
+    .endr
+    s_nop 4
+    MS_WIDE_SLAB_LOADS
+    s_add_u32 s84, s84, s85
+    s_nop 4
+    MS_WIDE_SLAB_LOADS
+    s_sub_u32 s84, s84, s85
+    s_waitcnt vmcnt(16)
+    s_barrier
+    .set ms_q, 0
+    .rept 16
+      MS_WIDE_READ ms_q, 128, 160, 112, 114
+      .set ms_q, ms_q+1
+    .endr
+  L_ms_wide_loop_%=:
+    s_waitcnt lgkmcnt(0)
+    MS_WIDE_STEP 128, 160, 192, 224, 113, 115, 0
+    v_add_u32 v112, s85, v112
+    v_add_u32 v113, s85, v113
+    v_add_u32 v114, s85, v114
+    v_add_u32 v115, s85, v115
+    s_waitcnt vmcnt(0) lgkmcnt(0)
+    s_barrier
+    s_cmp_gt_u32 s86, 2
+    s_cbranch_scc0 L_ms_wide_last_%=
+    MS_WIDE_STEP 192, 224, 128, 160, 112, 114, 1
+    s_add_u32 s80, s80, 128
+    s_addc_u32 s81, s81, 0
+    s_add_u32 s82, s82, 128
+    s_addc_u32 s83, s83, 0
+    s_branch L_ms_wide_join_%=
+  L_ms_wide_last_%=:
+    MS_WIDE_STEP 192, 224, 128, 160, 112, 114, 0
+  L_ms_wide_join_%=:
+    s_add_u32 s84, s84, s85
+    s_sub_u32 s85, 0, s85
+    s_sub_u32 s86, s86, 1
+    s_cmp_lg_u32 s86, 0
+    s_cbranch_scc1 L_ms_wide_loop_%=
+    s_waitcnt vmcnt(0) lgkmcnt(0)
+    s_nop 7
+    s_nop 7
+    s_nop 7
+    .purgem MS_WIDE_MFMA
+    .purgem MS_WIDE_READ
+    .purgem MS_WIDE_LOAD_TO
+    .purgem MS_WIDE_LOAD
+    .purgem MS_WIDE_SLAB_LOADS
+    .purgem MS_WIDE_STEP
+  )"
+               :
+               : [xo0] "v"(xo[0]), [xo1] "v"(xo[1]), [xo2] "v"(xo[2]), [xo3] "v"(xo[3]), [xo4] "v"(xo[4]), [xo5] "v"(xo[5]),
+                 [xo6] "v"(xo[6]), [xo7] "v"(xo[7]), [wo0] "v"(wo[0]), [wo1] "v"(wo[1]), [wo2] "v"(wo[2]), [wo3] "v"(wo[3]),
+                 [wo4] "v"(wo[4]), [wo5] "v"(wo[5]), [wo6] "v"(wo[6]), [wo7] "v"(wo[7]), [raw0] "v"(raw0), [raw1] "v"(raw1),
+                 [rax0] "v"(rax0), [rax1] "v"(rax1), [xb_lo] "s"(xb_lo), [xb_hi] "s"(xb_hi), [wb_lo] "s"(wb_lo),
+                 [wb_hi] "s"(wb_hi), [dma] "s"(dma), [slabs] "s"(slabs_left)
+               : "memory", "scc", "s80", "s81", "s82", "s83", "s84", "s85", "s86", MS_WIDE_VGPRS, MS_WIDE_AGPRS);
+
+  const bool vec_store = (ldc % 4 == 0);
+  // (gated: the output has N / 2 columns, and a lane's four of them are 8-byte aligned when ldc is a multiple of 4)
+  const bool inside = m0 + BM <= M && n0 + BN <= N && vec_store;
+  if (inside && (mode == 0 || mode >= 3) && ldc % 8 == 0 && (size_t)Cbase % 16 == 0) {
+    unsigned char* part = lds + wave * WIDE_STAGED_BYTES;
+    static_assert(MS_ACT_COUNT == 2, "one case per activation below");
+    if (mode == 0) wide_store_staged<0>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + n0 + wn, ldc, part, lane);
+    else if (mode == 3) wide_store_staged<3>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, part, lane);
+    else wide_store_staged<4>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, part, lane);
+    __syncthreads();  // the next item's loads go where other waves may still be reading their parts
+  } else if (inside) {
+    wide_epilogue<true>(C, Cbase, mode, m0 + wm + r, n0 + wn, g, M, N, ldc, vec_store);
+  } else {
+    wide_epilogue<false>(C, Cbase, mode, m0 + wm + r, n0 + wn, g, M, N, ldc, vec_store);
+  }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -547,19 +942,11 @@ extern "C" int ms_splitk_reduce(const float* P, void* C, int mode, int splits, i
 // bound by memory; with them at 850-950.
 constexpr long DMA_BAND_BYTES = 96L << 20;
 
-template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU, int WR = 2, int WC = 2>
-static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
-                      size_t stride, int splits, hipStream_t st) {
-  constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
-  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
-  if (!ready) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-      return MS_LAUNCH_FAILED;
-    ready = true;
-  }
-  const long blocks = (long)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
-  if (blocks > 0x7fffffffL) return MS_BAD_ARG;
+// How the blocks of a grid of BM x BN tiles walk it (the two last arguments of the kernels).
+struct TileWalk {
+  int xcd_rows, band_cols;
+};
+static TileWalk tile_walk(int M, int N, int K, int BM, int BN) {
   // How the XCDs share the tiles: as a grid of xcd_rows x 8 / xcd_rows rectangles where the tile counts
   // divide, chosen so that the bytes all XCDs read together (its share of the activations once per
   // XCD column, its share of the weights once per XCD row) are fewest, if that is under 0.6 of what
@@ -592,7 +979,60 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
     const long bands = (sub_cols + band_cols - 1) / band_cols;
     band_cols = (sub_cols + bands - 1) / bands;
   }
-  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC><<<(unsigned)blocks, WR * WC * WAVE, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, xcd_rows, (int)band_cols);
+  return TileWalk{xcd_rows, (int)band_cols};
+}
+
+template <int BM, int BN, int KS, int STAGES, int BLOCKS_PER_CU, int WR = 2, int WC = 2>
+static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
+                      size_t stride, int splits, hipStream_t st) {
+  constexpr int lds_bytes = STAGES * (BM + BN) * KS * 2;
+  static bool ready = false;  // more than 64 KB of LDS has to be asked for once per kernel
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  const long blocks = (long)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
+  if (blocks > 0x7fffffffL) return MS_BAD_ARG;
+  const TileWalk walk = tile_walk(M, N, K, BM, BN);
+  gemm_bf16_dma_kernel<BM, BN, KS, STAGES, BLOCKS_PER_CU, WR, WC><<<(unsigned)blocks, WR * WC * WAVE, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, walk.xcd_rows, walk.band_cols);
+  return launch_status();
+}
+
+// Compute units of the current device (asked once per device).
+static int compute_units() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n >= 8) ? n : 256;
+  }
+  return cached[dev];
+}
+
+// The 256 x 256 tile: four waves with the loop written out where every split has at least two slabs and a
+// tile's rows lie within 4 GB of its first (the loop adds 32-bit offsets to a tile's base), else eight waves.
+static int launch_256(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
+                      size_t stride, int splits, hipStream_t st) {
+  const int last_slabs = (K - (splits - 1) * k_per) / BK;  // of the last split, the shortest
+  if (last_slabs < 2 || k_per < 2 * BK || ldx >= (1 << 22) || K >= (1 << 22))
+    return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+  constexpr int lds_bytes = 4 * WIDE_STAGED_BYTES;  // the loop's two stages are 128 KB of it
+  static_assert(lds_bytes >= 2 * (256 + 256) * BK * 2 && lds_bytes <= 160 * 1024, "LDS of the wide tile");
+  static bool ready = false;
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  const long items = (long)((N + 255) / 256) * ((M + 255) / 256) * splits;
+  if (items > 0x7fffffffL) return MS_BAD_ARG;
+  const TileWalk walk = tile_walk(M, N, K, 256, 256);
+  const int cus = compute_units();
+  const int blocks = items <= cus ? (int)items : cus / 8 * 8;
+  gemm_bf16_wide_kernel<<<(unsigned)blocks, 256, lds_bytes, st>>>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, walk.xcd_rows, walk.band_cols, (int)items);
   return launch_status();
 }
 
@@ -647,7 +1087,7 @@ static int pick_tile_cols(int M, int N, int K, int splits, bool pairs, float* pr
 static int launch_picked(int cols, const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc,
                          int k_per, size_t stride, int splits, hipStream_t st) {
   switch (cols) {
-    case 256: return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    case 256: return launch_256(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     case 192: return launch_dma<128, 192, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     case 160: return launch_dma<128, 160, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
     case 64: return launch_dma<128, 64, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
