@@ -86,6 +86,89 @@ __device__ __forceinline__ float activate_fast(float x, int act) {
   return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
+// Four consecutive n of row m: the store of one accumulator fragment. MODE 0: bf16, 1: float, 2: float +=.
+// INSIDE: the tile's columns lie within the matrix and a lane's four are aligned for one store, so only
+// the row is tested (a ragged last row of tiles, which any token count makes, runs the same code as the rest:
+// code that only a few blocks run is not in the instruction cache when they get there).
+template <int MODE, bool INSIDE>
+__device__ __forceinline__ void store_fragment(void* __restrict__ C, int m, int n, int M, int N, int ldc, floatx4 a, bool vec_ok) {
+  if constexpr (!INSIDE) {
+    store4(C, MODE, m, n, M, N, ldc, a, vec_ok);
+  } else {
+    if (m >= M) return;
+    const size_t at = (size_t)m * ldc + n;
+    if constexpr (MODE == 0) {
+      union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.e[i] = static_cast<bf16>(a[i]);
+      *reinterpret_cast<uint2*>((bf16*)C + at) = o.u;
+    } else if constexpr (MODE == 1) {
+      *reinterpret_cast<float4*>((float*)C + at) = make_float4(a[0], a[1], a[2], a[3]);
+    } else {
+      float4 c = *reinterpret_cast<float4*>((float*)C + at);
+      c.x += a[0]; c.y += a[1]; c.z += a[2]; c.w += a[3];
+      *reinterpret_cast<float4*>((float*)C + at) = c;
+    }
+  }
+}
+
+// Gate and up fragments of the same four outputs (W holds alternating blocks of 16 gate rows and 16 up
+// rows): out[m, col ..] = act(gate) * up, bf16 with row stride ldc; `half` = N / 2 columns.
+template <int ACT, bool INSIDE>
+__device__ __forceinline__ void store_gated(bf16* __restrict__ out, int m, int col, int M, int half, int ldc, floatx4 gate, floatx4 up) {
+  if (m >= M || (!INSIDE && col >= half)) return;
+  union { uint2 u; bf16 e[4]; } o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(activate_fast(gate[e], ACT) * up[e]);
+  *reinterpret_cast<uint2*>(out + (size_t)m * ldc + col) = o.u;
+}
+
+// A wave tile's accumulators acc[i][j] (i: block of 16 n, j: block of 16 m) to memory. m, n: this lane's
+// row and first column in fragment (0, 0). MODE as above (3 + activation: gated, C unused).
+template <int MODE, bool INSIDE, int FN, int FM>
+__device__ __forceinline__ void store_fragments(const floatx4 (&acc)[FN][FM], void* C, void* Cbase, int m, int n, int M, int N, int ldc,
+                                                bool vec_store) {
+  if constexpr (MODE >= 3) {
+    const int g4 = n % 16;  // the lane's group of four columns
+#pragma unroll
+    for (int i = 0; i + 1 < FN; i += 2)
+#pragma unroll
+      for (int j = 0; j < FM; ++j)
+        store_gated<MODE - 3, INSIDE>((bf16*)Cbase, m + j * 16, (n - g4 + i * 16) / 2 + g4, M, N / 2, ldc, acc[i][j], acc[i + 1][j]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < FN; ++i)
+#pragma unroll
+      for (int j = 0; j < FM; ++j) store_fragment<MODE, INSIDE>(C, m + j * 16, n + i * 16, M, N, ldc, acc[i][j], vec_store);
+  }
+}
+
+// The same into a tile image in LDS as bfloat16 (MODE 0, or 3 + activation: gated). at: this lane's place
+// in fragment (0, 0); row_bytes: stride of the image's rows.
+template <int MODE, int FN, int FM>
+__device__ __forceinline__ void stage_fragments(const floatx4 (&acc)[FN][FM], unsigned char* at, int row_bytes) {
+  union { uint2 u; bf16 e[4]; } o;
+  if constexpr (MODE >= 3) {
+#pragma unroll
+    for (int i = 0; i + 1 < FN; i += 2)
+#pragma unroll
+      for (int j = 0; j < FM; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(activate_fast(acc[i][j][e], MODE - 3) * acc[i + 1][j][e]);
+        *reinterpret_cast<uint2*>(at + j * 16 * row_bytes + (i / 2) * 32) = o.u;
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < FN; ++i)
+#pragma unroll
+      for (int j = 0; j < FM; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(acc[i][j][e]);
+        *reinterpret_cast<uint2*>(at + j * 16 * row_bytes + i * 32) = o.u;
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Tile kernel.
 #define BK 64
@@ -357,34 +440,56 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
         for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
   }
 
-  if (mode >= 3) {
-    // Gated epilogue (mode 3 + an MS_ACT_* number): W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and
-    // 2 p + 1 of a lane are gate and up of the same four outputs: out[m, n / 2 ...] = act(gate) * up,
-    // bf16 [M, N / 2] with row stride ldc. Wave tiles with an odd number of fragments are never
-    // launched in this mode.
-#pragma unroll
-    for (int i = 0; i + 1 < FN; i += 2)
-#pragma unroll
-      for (int j = 0; j < FM; ++j) {
-        const int m = m0 + wm + j * 16 + r, col = (n0 + wn + i * 16) / 2 + g * 4;
-        if (m < M && col < N / 2) {
-          union { uint2 u; bf16 e[4]; } o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float gate = acc[i][j][e];
-            o.e[e] = static_cast<bf16>(activate(gate, mode - 3) * acc[i + 1][j][e]);
-          }
-          *reinterpret_cast<uint2*>((bf16*)Cbase + (size_t)m * ldc + col) = o.u;
-        }
-      }
+  // Epilogue. Modes 0 to 2 store the fragments as they are. Mode 3 + an MS_ACT_* number is the gated one:
+  // W holds alternating blocks of 16 gate rows and 16 up rows, so fragments 2 p and 2 p + 1 of a lane are
+  // gate and up of the same four outputs: out[m, n / 2 ...] = act(gate) * up, bf16 [M, N / 2] with row
+  // stride ldc (wave tiles with an odd number of fragments are never launched in this mode). The mode is
+  // told apart once, not per fragment, so that each mode's stores are one straight run of code: with the
+  // test inside, a tile's epilogue jumped through a hundred kilobytes of code the instruction cache had
+  // never seen, which took longer than ten slabs of products.
+  const bool vec_store = (ldc % 4 == 0);
+  const bool inside = n0 + BN <= N && vec_store;  // the columns; rows are tested where they are stored
+  // bfloat16 outputs of a tile whose columns lie inside the matrix, rows 16-byte aligned, go through LDS
+  // (the ring is free after the loop): a lane's four values of a row into a padded row of the tile
+  // (conflict-free), then every thread takes 16 bytes of a row, so that store instructions write whole
+  // 128-byte lines instead of 32-byte pieces of sixteen rows each, which cost the L2 four times the requests.
+  constexpr int OUT_ROW = BN * 2 + 16, GATED_ROW = BN + 16;
+  if (inside && ldc % 8 == 0 && (size_t)Cbase % 16 == 0 &&
+      ((mode == 0 && BM * OUT_ROW <= STAGES * STAGE_BYTES) || (mode >= 3 && BM * GATED_ROW <= STAGES * STAGE_BYTES))) {
+    __syncthreads();  // every wave has read the last slab's fragments
+    const int row_bytes = mode == 0 ? OUT_ROW : GATED_ROW;
+    static_assert(MS_ACT_COUNT == 2, "one case per activation below");
+    if (mode == 0) stage_fragments<0, FN, FM>(acc, lds + (wm + r) * OUT_ROW + (wn + g * 4) * 2, OUT_ROW);
+    else if (mode == 3) stage_fragments<3, FN, FM>(acc, lds + (wm + r) * GATED_ROW + (wn / 2 + g * 4) * 2, GATED_ROW);
+    else stage_fragments<4, FN, FM>(acc, lds + (wm + r) * GATED_ROW + (wn / 2 + g * 4) * 2, GATED_ROW);
+    __syncthreads();
+    const int chunks = (row_bytes - 16) / 16;  // 16-byte chunks of an output row of the tile
+    bf16* out = (bf16*)Cbase + (size_t)m0 * ldc + (mode == 0 ? n0 : n0 / 2);
+    for (int c = tid; c < BM * chunks; c += NW * WAVE) {
+      const int row = c / chunks, ch = c % chunks;
+      if (m0 + row < M)
+        *reinterpret_cast<uint4*>(out + (size_t)row * ldc + ch * 8) = *reinterpret_cast<const uint4*>(lds + row * row_bytes + ch * 16);
+    }
     return;
   }
-  const bool vec_store = (ldc % 4 == 0);
-#pragma unroll
-  for (int i = 0; i < FN; ++i)
-#pragma unroll
-    for (int j = 0; j < FM; ++j)
-      store4(C, mode, m0 + wm + j * 16 + r, n0 + wn + i * 16 + g * 4, M, N, ldc, acc[i][j], vec_store);
+  const int m = m0 + wm + r, n = n0 + wn + g * 4;
+  if (inside) {
+    switch (mode) {
+      case 0: store_fragments<0, true, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 1: store_fragments<1, true, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 2: store_fragments<2, true, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 3: store_fragments<3, true, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      default: store_fragments<4, true, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+    }
+  } else {
+    switch (mode) {
+      case 0: store_fragments<0, false, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 1: store_fragments<1, false, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 2: store_fragments<2, false, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      case 3: store_fragments<3, false, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+      default: store_fragments<4, false, FN, FM>(acc, C, Cbase, m, n, M, N, ldc, vec_store); break;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -424,40 +529,6 @@ __device__ __forceinline__ floatx4 wide_acc() {
   return v;
 }
 
-// Four consecutive n of row m: the store of one accumulator fragment. MODE 0: bf16, 1: float, 2: float +=.
-// INSIDE: the tile lies wholly within the matrix and rows are 8-byte aligned, so nothing is tested.
-template <int MODE, bool INSIDE>
-__device__ __forceinline__ void store_fragment(void* __restrict__ C, int m, int n, int M, int N, int ldc, floatx4 a, bool vec_ok) {
-  if constexpr (!INSIDE) {
-    store4(C, MODE, m, n, M, N, ldc, a, vec_ok);
-  } else {
-    const size_t at = (size_t)m * ldc + n;
-    if constexpr (MODE == 0) {
-      union { uint2 u; bf16 e[4]; } o;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o.e[i] = static_cast<bf16>(a[i]);
-      *reinterpret_cast<uint2*>((bf16*)C + at) = o.u;
-    } else if constexpr (MODE == 1) {
-      *reinterpret_cast<float4*>((float*)C + at) = make_float4(a[0], a[1], a[2], a[3]);
-    } else {
-      float4 c = *reinterpret_cast<float4*>((float*)C + at);
-      c.x += a[0]; c.y += a[1]; c.z += a[2]; c.w += a[3];
-      *reinterpret_cast<float4*>((float*)C + at) = c;
-    }
-  }
-}
-
-// Gate and up fragments of the same four outputs (W holds alternating blocks of 16 gate rows and 16 up
-// rows): out[m, col ..] = act(gate) * up, bf16 with row stride ldc; `half` = N / 2 columns.
-template <int ACT, bool INSIDE>
-__device__ __forceinline__ void store_gated(bf16* __restrict__ out, int m, int col, int M, int half, int ldc, floatx4 gate, floatx4 up) {
-  if (!INSIDE && (m >= M || col >= half)) return;
-  union { uint2 u; bf16 e[4]; } o;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) o.e[e] = static_cast<bf16>(activate_fast(gate[e], ACT) * up[e]);
-  *reinterpret_cast<uint2*>(out + (size_t)m * ldc + col) = o.u;
-}
-
 // Fragments (2 P, J) and (2 P + 1, J) of the wide tile. MODE 0 to 2: stored as they are; 3 + an MS_ACT_*
 // number: as gate and up. m: this lane's row in row block 0; nb: the wave tile's first column; g: the
 // lane's group of four columns.
@@ -479,8 +550,8 @@ __device__ __forceinline__ void wide_stores(std::integer_sequence<int, I...>, vo
   (wide_store<MODE, INSIDE, I / 8, I % 8>(C, Cbase, m, nb, g, M, N, ldc, vec_store), ...);
 }
 
-// The same through LDS, for bfloat16 outputs of tiles that lie wholly inside the matrix with 16-byte
-// aligned rows: a lane's four values of a row go into the wave's own part of LDS (rows padded by 16
+// The same through LDS, for bfloat16 outputs of tiles whose columns lie inside the matrix, with 16-byte
+// aligned rows (`rows` of the wave tile's 128 exist): a lane's four values of a row go into the wave's own part of LDS (rows padded by 16
 // bytes: conflict-free), then every lane takes 16 bytes of a row back, so that a store instruction
 // writes whole 128-byte lines (four rows' worth) instead of 32-byte pieces of sixteen rows. The pieces
 // cost four times the requests at the L2, and a tile's stores then took as long as ten slabs of products.
@@ -510,7 +581,7 @@ __device__ __forceinline__ void wide_stage_all(std::integer_sequence<int, I...>,
 }
 // out: the wave tile's first output element; MODE 0 or 3 + an MS_ACT_* number.
 template <int MODE>
-__device__ __forceinline__ void wide_store_staged(bf16* __restrict__ out, int ldc, unsigned char* part, int lane) {
+__device__ __forceinline__ void wide_store_staged(bf16* __restrict__ out, int ldc, int rows, unsigned char* part, int lane) {
   wide_stage_all<MODE>(std::make_integer_sequence<int, 32>{}, part, lane % 16, lane / 16);
   constexpr int CHUNKS = MODE >= 3 ? 8 : 16, STRIDE = CHUNKS * 16 + 16, ROWS = 64 / CHUNKS;
   const int lrow = lane / CHUNKS, ch = lane % CHUNKS;
@@ -518,7 +589,7 @@ __device__ __forceinline__ void wide_store_staged(bf16* __restrict__ out, int ld
   for (int it = 0; it < 128 / ROWS; ++it) {
     const int row = it * ROWS + lrow;
     const uint4 v = *reinterpret_cast<const uint4*>(part + row * STRIDE + ch * 16);
-    *reinterpret_cast<uint4*>(out + (size_t)row * ldc + ch * 8) = v;
+    if (row < rows) *reinterpret_cast<uint4*>(out + (size_t)row * ldc + ch * 8) = v;
   }
 }
 
@@ -749,13 +820,14 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
 
   const bool vec_store = (ldc % 4 == 0);
   // (gated: the output has N / 2 columns, and a lane's four of them are 8-byte aligned when ldc is a multiple of 4)
-  const bool inside = m0 + BM <= M && n0 + BN <= N && vec_store;
+  const bool inside = n0 + BN <= N && vec_store;  // the columns; rows are tested where they are stored
   if (inside && (mode == 0 || mode >= 3) && ldc % 8 == 0 && (size_t)Cbase % 16 == 0) {
     unsigned char* part = lds + wave * WIDE_STAGED_BYTES;
+    const int rows = M - (m0 + wm);  // of the wave tile's 128 that exist
     static_assert(MS_ACT_COUNT == 2, "one case per activation below");
-    if (mode == 0) wide_store_staged<0>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + n0 + wn, ldc, part, lane);
-    else if (mode == 3) wide_store_staged<3>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, part, lane);
-    else wide_store_staged<4>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, part, lane);
+    if (mode == 0) wide_store_staged<0>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + n0 + wn, ldc, rows, part, lane);
+    else if (mode == 3) wide_store_staged<3>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane);
+    else wide_store_staged<4>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane);
     __syncthreads();  // the next item's loads go where other waves may still be reading their parts
   } else if (inside) {
     wide_epilogue<true>(C, Cbase, mode, m0 + wm + r, n0 + wn, g, M, N, ldc, vec_store);
@@ -1013,12 +1085,12 @@ static int compute_units() {
 }
 
 // The 256 x 256 tile: four waves with the loop written out where every split has at least two slabs and a
-// tile's rows lie within 4 GB of its first (the loop adds 32-bit offsets to a tile's base), else eight waves.
+// tile's rows lie within 4 GB of its first (the loop adds 32-bit offsets to a tile's base), else 128 x 128 tiles.
 static int launch_256(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
                       size_t stride, int splits, hipStream_t st) {
   const int last_slabs = (K - (splits - 1) * k_per) / BK;  // of the last split, the shortest
   if (last_slabs < 2 || k_per < 2 * BK || ldx >= (1 << 22) || K >= (1 << 22))
-    return launch_dma<256, 256, BK, 2, 1, 4, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
+    return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
   constexpr int lds_bytes = 4 * WIDE_STAGED_BYTES;  // the loop's two stages are 128 KB of it
   static_assert(lds_bytes >= 2 * (256 + 256) * BK * 2 && lds_bytes <= 160 * 1024, "LDS of the wide tile");
   static bool ready = false;
