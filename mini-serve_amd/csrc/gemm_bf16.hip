@@ -626,7 +626,6 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // 2 * STAGE_BYTES, and 4 * WIDE_STAGED_BYTES for the stores
 
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  const int r = lane % 16, g = lane / 16;
   const int wm = (wave / 2) * 128, wn = (wave % 2) * 128;
   // A block works through items blockIdx.x, + gridDim.x, ...: one block per CU stays for the whole product, so
   // that a tile's stores drain and the next tile's first loads fly while no block has to end and another
@@ -659,11 +658,11 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
   const unsigned dma = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * 8192u);
   // Read side: the rows of a fragment are base + r with base a multiple of 16, so the slot of chunk c
   // is c ^ (r >> 1) for every fragment; step t reads chunk column 4 t + g.
-  const unsigned sw = (unsigned)(r >> 1) & 7u;
-  const unsigned raw0 = lds0 + BM * ROW_BYTES + (unsigned)(wn + r) * ROW_BYTES + (((unsigned)g ^ sw) * 16u);
-  const unsigned raw1 = lds0 + BM * ROW_BYTES + (unsigned)(wn + r) * ROW_BYTES + (((unsigned)(4 + g) ^ sw) * 16u);
-  const unsigned rax0 = lds0 + (unsigned)(wm + r) * ROW_BYTES + (((unsigned)g ^ sw) * 16u);
-  const unsigned rax1 = lds0 + (unsigned)(wm + r) * ROW_BYTES + (((unsigned)(4 + g) ^ sw) * 16u);
+  const unsigned fr = (unsigned)lane % 16u, fg = (unsigned)lane / 16u, sw = (fr >> 1) & 7u;
+  const unsigned raw0 = lds0 + BM * ROW_BYTES + ((unsigned)wn + fr) * ROW_BYTES + ((fg ^ sw) * 16u);
+  const unsigned raw1 = lds0 + BM * ROW_BYTES + ((unsigned)wn + fr) * ROW_BYTES + (((4u + fg) ^ sw) * 16u);
+  const unsigned rax0 = lds0 + ((unsigned)wm + fr) * ROW_BYTES + ((fg ^ sw) * 16u);
+  const unsigned rax1 = lds0 + ((unsigned)wm + fr) * ROW_BYTES + (((4u + fg) ^ sw) * 16u);
 
 // Between the 64 products of a step: a fragment read after every third (all 16 are out 18 products
 // before the step ends, so the next step starts without waiting for them), a load into LDS after every
@@ -818,6 +817,12 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
                  [wb_hi] "s"(wb_hi), [dma] "s"(dma), [slabs] "s"(slabs_left)
                : "memory", "scc", "s80", "s81", "s82", "s83", "s84", "s85", "s86", MS_WIDE_VGPRS, MS_WIDE_AGPRS);
 
+  // The stores' address arithmetic starts from a lane number the compiler cannot see through: what
+  // it could work out once for all items it would keep in registers across the loop, of which it has 96
+  // there, and spill.
+  int lane_now = lane;
+  asm volatile("" : "+v"(lane_now));
+  const int r = lane_now % 16, g = lane_now / 16;
   const bool vec_store = (ldc % 4 == 0);
   // (gated: the output has N / 2 columns, and a lane's four of them are 8-byte aligned when ldc is a multiple of 4)
   const bool inside = n0 + BN <= N && vec_store;  // the columns; rows are tested where they are stored
@@ -825,9 +830,9 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
     unsigned char* part = lds + wave * WIDE_STAGED_BYTES;
     const int rows = M - (m0 + wm);  // of the wave tile's 128 that exist
     static_assert(MS_ACT_COUNT == 2, "one case per activation below");
-    if (mode == 0) wide_store_staged<0>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + n0 + wn, ldc, rows, part, lane);
-    else if (mode == 3) wide_store_staged<3>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane);
-    else wide_store_staged<4>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane);
+    if (mode == 0) wide_store_staged<0>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + n0 + wn, ldc, rows, part, lane_now);
+    else if (mode == 3) wide_store_staged<3>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane_now);
+    else wide_store_staged<4>((bf16*)Cbase + (size_t)(m0 + wm) * ldc + (n0 + wn) / 2, ldc, rows, part, lane_now);
     __syncthreads();  // the next item's loads go where other waves may still be reading their parts
   } else if (inside) {
     wide_epilogue<true>(C, Cbase, mode, m0 + wm + r, n0 + wn, g, M, N, ldc, vec_store);
@@ -1072,6 +1077,9 @@ static int launch_dma(const bf16* x, const bf16* w, void* C, int mode, int M, in
   return launch_status();
 }
 
+// The wide tile's loop adds 32-bit byte offsets of up to 255 rows to a tile's base.
+static bool wide_tile_offsets_fit(int ldx, int K) { return ldx < (1 << 22) && K < (1 << 22); }
+
 // Compute units of the current device (asked once per device).
 static int compute_units() {
   static int cached[64];
@@ -1089,7 +1097,7 @@ static int compute_units() {
 static int launch_256(const bf16* x, const bf16* w, void* C, int mode, int M, int N, int K, int ldx, int ldc, int k_per,
                       size_t stride, int splits, hipStream_t st) {
   const int last_slabs = (K - (splits - 1) * k_per) / BK;  // of the last split, the shortest
-  if (last_slabs < 2 || k_per < 2 * BK || ldx >= (1 << 22) || K >= (1 << 22))
+  if (last_slabs < 2 || k_per < 2 * BK || !wide_tile_offsets_fit(ldx, K))
     return launch_dma<128, 128, BK, 2, 2>(x, w, C, mode, M, N, K, ldx, ldc, k_per, stride, splits, st);
   constexpr int lds_bytes = 4 * WIDE_STAGED_BYTES;  // the loop's two stages are 128 KB of it
   static_assert(lds_bytes >= 2 * (256 + 256) * BK * 2 && lds_bytes <= 160 * 1024, "LDS of the wide tile");
@@ -1109,24 +1117,35 @@ static int launch_256(const bf16* x, const bf16* w, void* C, int mode, int M, in
 }
 
 // Tile shape of a product with at least 256 tiles of 128 x 128: 128-row tiles of four waves, 64 to 192
-// columns wide, two blocks per CU (512 run at once), or 256 x 256 tiles of eight waves (4 x 2, wave
-// tiles of 64 x 128, one block per CU with all 256 registers and 128 KB of LDS: a wave reads 12
-// fragments for 32 products where the 64 x 64 wave tile reads 8 for 16). The choice is the least
-// predicted time: a fixed part (launch, first slab, stores) plus, per slab of 64 k, the time of a round
-// of blocks. A block that has a CU to itself is faster than one that shares it, so a last round of up
-// to 256 blocks counts less than a full one. The figures (microseconds) are a fit to 270 products
-// (384 to 8,192 rows, 1,024 to 24,576 columns, K of 1,024, 4,096 and 12,288) timed with every shape;
-// picking by them is within 1 % of the best shape on average and 17 % at worst, where rules by tile
-// counts alone lost up to 28 % (2,048 x 5,120 x 12,288: 160 columns make exactly 512 tiles).
+// columns wide, two blocks per CU (512 run at once), or 256 x 256 tiles of four waves with wave tiles of
+// 128 x 128 (one block per CU that stays and takes tiles in turn; a wave reads 16 fragments for 64
+// products where the 64 x 64 wave tile reads 8 for 16). The choice is the least predicted time. For
+// the 128-row tiles: a fixed part (launch, first slab, stores) plus, per slab of 64 k, the time of a
+// round of blocks; a block that has a CU to itself is faster than one that shares it, so a last round
+// of up to 256 blocks counts less than a full one. For the 256 x 256 tile: a fixed part per launch and,
+// per round of 256 tiles, another (first slab, stores) plus its slabs, a last round of up to 128 tiles counting less per slab (half
+// the chip idles: less traffic). The figures (microseconds) are fits to products of 384 to 8,192 rows,
+// 1,024 to 24,576 columns and K of 1,024, 4,096 and 12,288 timed with every shape (270 for the 128-row
+// tiles, 177 for the 256 x 256 tile as it is now); over those 177 picking by them takes 0.5 % longer
+// in total than the best shape of each, 1.2 % per product on average and 29 % at worst, where rules by
+// tile counts alone lost up to 28 % in whole layers (2,048 x 5,120 x 12,288: 160 columns make exactly
+// 512 tiles).
 struct TileShape {
   int cols;      // 256 stands for the 256 x 256 tile
   float fixed;   // per launch
-  float alone;   // per slab, a last round with one block per CU
-  float shared;  // per slab, a round with two blocks per CU
+  float alone;   // per slab, a last round with one block per CU (256: with up to 128 tiles)
+  float shared;  // per slab, a round with two blocks per CU (256: any other round)
+  float round;   // per round of tiles (256 only)
 };
 static const TileShape TILE_SHAPES[5] = {
-    {128, 7.7f, 0.611f, 0.976f}, {64, 6.1f, 0.456f, 0.627f}, {160, 8.8f, 0.707f, 1.168f},
-    {192, 9.1f, 0.803f, 1.364f}, {256, 12.6f, 1.476f, 1.476f}};
+    {128, 7.7f, 0.611f, 0.976f, 0.f}, {64, 6.1f, 0.456f, 0.627f, 0.f}, {160, 8.8f, 0.707f, 1.168f, 0.f},
+    {192, 9.1f, 0.803f, 1.364f, 0.f}, {256, 4.5f, 0.997f, 1.306f, 3.9f}};
+
+// Whether the 256 x 256 tile takes a product of this K in this many splits: its loop needs two slabs.
+static bool wide_tile_runs(int K, int splits) {
+  const int slabs = (K + BK - 1) / BK, per = (slabs + splits - 1) / splits;
+  return per >= 2 && slabs - (splits - 1) * per >= 2;
+}
 
 // `pairs`: the gated epilogue needs an even number of 16-column fragments per wave, which 160 columns
 // over two waves are not.
@@ -1137,16 +1156,18 @@ static int pick_tile_cols(int M, int N, int K, int splits, bool pairs, float* pr
   for (int i = 0; i < 5; ++i) {
     const TileShape& t = TILE_SHAPES[i];
     if (pairs && t.cols == 160) continue;
-    float rounds;
+    float time;
     if (t.cols == 256) {
       const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256) * splits;
-      rounds = (float)((tiles + 255) / 256) * t.shared;
+      const long rest = tiles % 256;
+      if (!wide_tile_runs(K, splits)) continue;
+      time = t.fixed + (float)(tiles / 256) * (t.round + slabs * t.shared) +
+             (rest == 0 ? 0.f : t.round + slabs * (rest <= 128 ? t.alone : t.shared));
     } else {
       const long tiles = (long)((M + 127) / 128) * ((N + t.cols - 1) / t.cols) * splits;
       const long rest = tiles % 512;
-      rounds = (float)(tiles / 512) * t.shared + (rest == 0 ? 0.f : rest <= 256 ? t.alone : t.shared);
+      time = t.fixed + slabs * ((float)(tiles / 512) * t.shared + (rest == 0 ? 0.f : rest <= 256 ? t.alone : t.shared));
     }
-    const float time = t.fixed + slabs * rounds;
     if (i == 0 || time < least) {
       least = time;
       best = t.cols;
@@ -1441,7 +1462,8 @@ extern "C" int ms_gemm_bf16_tile_shape(int M, int N, int K, int ldx, int splits,
   const long big = (long)((M + 127) / 128) * ((N + 127) / 128) * splits;
   if (big < 256) return 64064;
   const int cols = pick_tile_cols(M, N, K, splits, gated != 0);
-  return cols == 256 ? 256256 : 128000 + cols;
+  if (cols == 256) return wide_tile_offsets_fit(ldx, K) ? 256256 : 128128;
+  return 128000 + cols;
 }
 
 // mode 0: C bf16 = X W^T   mode 1: C float = X W^T   mode 2: C float += X W^T

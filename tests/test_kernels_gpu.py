@@ -134,10 +134,10 @@ def test_act_mul(ops, dtype, inter, act):
 # run the product and the activation as two kernels. All must agree.
 GATED = [(3000, 128, 4096), (1, 1024, 3072), (8, 1024, 3072), (16, 512, 64), (5, 2048, 160), (13, 4096, 48), (40, 1024, 3072), (64, 256, 64),
          (17, 1024, 3072), (32, 768, 160), (33, 512, 48), (64, 1024, 3072), (50, 2048, 64),
-         (200, 1024, 3072), (2048, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096),
+         (200, 1024, 3072), (2048, 1024, 3072), (1000, 1024, 3072), (300, 192, 8192), (130, 96, 224), (9, 100, 48), (3000, 64, 4096),
          (2048, 512, 12288), (4090, 512, 4080)]
 # The tile the activation's epilogue runs in, for the rows that are here for one (None: not asserted).
-GATED_TILES = {(3000, 128, 4096): (128, 128), (200, 1024, 3072): (64, 64), (2048, 1024, 3072): (128, 192),
+GATED_TILES = {(3000, 128, 4096): (128, 128), (200, 1024, 3072): (64, 64), (2048, 1024, 3072): (256, 256), (1000, 1024, 3072): (128, 192),
                (300, 192, 8192): (128, 64), (3000, 64, 4096): (128, 64),
                (2048, 512, 12288): (256, 256), (4090, 512, 4080): (256, 256)}  # the last: ragged in both directions
 
@@ -207,8 +207,10 @@ def test_gemm_bf16(ops, m, n, k):
     (1990, 5100, 512, (128, 160)), (4100, 1000, 512, (128, 160)),
     # 128 x 192 (many rows, and few rows of a wide matrix)
     (4000, 4200, 1024, (128, 192)), (600, 33000, 512, (128, 192)),
-    # 256 x 256 tiles of eight waves (exactly one round of 256 with both edges ragged, and 240 tiles)
+    # 256 x 256 tiles of four waves, one block per CU taking tiles in turn (exactly 256 with both edges ragged, and 240 tiles)
     (4090, 4090, 1024, (256, 256)), (3000, 5000, 1024, (256, 256)),
+    # the same with the fewest slabs its loop takes (two), with three, and two rounds of tiles with five slabs
+    (4000, 4088, 128, (256, 256)), (2048, 8192, 192, (256, 256)), (4096, 8192, 320, (256, 256)),
 ])
 def test_gemm_bf16_large_tiles(ops, m, n, k, tile):
     """Every tile shape of the kernel whose slabs go straight into LDS (K a multiple of 64). Which shape a
@@ -287,10 +289,12 @@ def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
 
 @pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 8), (2048, 1024, 3072, 2), (300, 1000, 1100, 6), (2048, 4096, 1024, 1),
                                           (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6),
-                                          (1024, 4096, 12288, 2), (768, 5120, 8192, 2)])
+                                          (1024, 4096, 12288, 4), (768, 5120, 8192, 4), (2048, 4096, 8384, 2), (4000, 2048, 8256, 2)])
 def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
-    """The last two have 256 and more tiles of 128 x 128 already: above 512 rows the splits follow the
-    predicted time (a long K in two halves fills two blocks per CU), not the tile count alone."""
+    """The last four have 256 and more tiles of 128 x 128 already: above 512 rows the splits follow the
+    predicted time (a long K in parts makes 256 x 256 tiles enough to give every CU one), not the tile
+    count alone. The very last two have a last split that is one slab shorter than the others, with an
+    odd and an even number of slabs."""
     x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
     want = x.double() @ w.double().T
     resid = rand((m, n), F32, 62)
