@@ -665,15 +665,17 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
   const unsigned rax1 = lds0 + ((unsigned)wm + fr) * ROW_BYTES + (((4u + fg) ^ sw) * 16u);
 
 // Between the 64 products of a step: a fragment read after every third (all 16 are out 18 products
-// before the step ends, so the next step starts without waiting for them), a load into LDS after every
-// fourth (all 16 at once, right after the barrier, measured 11 % slower: the loads' LDS writes then
-// crowd out the fragment reads).
-#define MS_WIDE_READ_EVERY 3
+// before the step ends, so the next step starts without waiting for them; every second or fourth
+// measured the same), a load into LDS around every fourth. The loads are best spread as thin as a step
+// allows: every third measured 3 % slower, every second in either half of the step 7 %, all 16 right after
+// the barrier 11 to 12 %: their LDS writes then crowd out the fragment reads.
+#define MS_WIDE_READ_EVERY 3  // a fragment read after products 1, 4, 7, ... of a step
 #define MS_WIDE_READ_FIRST 1
-#define MS_WIDE_LOAD_EVERY 4
+#define MS_WIDE_LOAD_EVERY 4  // a load into LDS around products 3, 7, 11, ... of a slab's second step
+#define MS_WIDE_LOAD_FIRST 3
 #define MS_STR2(x) #x
 #define MS_STR(x) MS_STR2(x)
-  asm volatile(".set ms_read_every, " MS_STR(MS_WIDE_READ_EVERY) "\n.set ms_read_first, " MS_STR(MS_WIDE_READ_FIRST) "\n.set ms_load_every, " MS_STR(MS_WIDE_LOAD_EVERY) "\n" R"(
+  asm volatile(".set ms_read_every, " MS_STR(MS_WIDE_READ_EVERY) "\n.set ms_read_first, " MS_STR(MS_WIDE_READ_FIRST) "\n.set ms_load_every, " MS_STR(MS_WIDE_LOAD_EVERY) "\n.set ms_load_first, " MS_STR(MS_WIDE_LOAD_FIRST) "\n" R"(
     .macro MS_WIDE_MFMA mi, cw, cx
       v_mfma_f32_16x16x32_bf16 a[(\mi)*4:(\mi)*4+3], v[\cw+((\mi)>>3)*4:\cw+((\mi)>>3)*4+3], v[\cx+((\mi)&7)*4:\cx+((\mi)&7)*4+3], a[(\mi)*4:(\mi)*4+3]
     .endm
@@ -710,19 +712,17 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
     .macro MS_WIDE_STEP cw, cx, nw, nx, aw, ax, loads
       .set ms_mi, 0
       .rept 64
-        .if \loads
-          .if ((ms_mi-(ms_mi/ms_load_every)*ms_load_every) == ms_load_every-1) && ((ms_mi/ms_load_every) < 16)
-            MS_WIDE_LOAD_TO (ms_mi/ms_load_every)
-          .endif
+        .set ms_rq, (ms_mi-ms_read_first)/ms_read_every
+        .set ms_lq, (ms_mi-ms_load_first)/ms_load_every
+        .if \loads && (ms_mi >= ms_load_first) && ((ms_mi-ms_load_first) == ms_lq*ms_load_every) && (ms_lq < 16)
+          MS_WIDE_LOAD_TO ms_lq
         .endif
         MS_WIDE_MFMA ms_mi, \cw, \cx
-        .if ((ms_mi-(ms_mi/ms_read_every)*ms_read_every) == ms_read_first) && ((ms_mi/ms_read_every) < 16)
-          MS_WIDE_READ (ms_mi/ms_read_every), \nw, \nx, \aw, \ax
+        .if (ms_mi >= ms_read_first) && ((ms_mi-ms_read_first) == ms_rq*ms_read_every) && (ms_rq < 16)
+          MS_WIDE_READ ms_rq, \nw, \nx, \aw, \ax
         .endif
-        .if \loads
-          .if ((ms_mi-(ms_mi/ms_load_every)*ms_load_every) == ms_load_every-1) && ((ms_mi/ms_load_every) < 16)
-            MS_WIDE_LOAD (ms_mi/ms_load_every)
-          .endif
+        .if \loads && (ms_mi >= ms_load_first) && ((ms_mi-ms_load_first) == ms_lq*ms_load_every) && (ms_lq < 16)
+          MS_WIDE_LOAD ms_lq
         .endif
         .set ms_mi, ms_mi+1
       .endr
@@ -755,17 +755,17 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_wide_kernel(const bf16* __re
     s_mov_b32 s84, %[dma]
     s_mov_b32 s85, 0x10000
     s_mov_b32 s86, %[slabs]
-    .set ms_q, 0
-    .rept 256
-      v_accvgpr_write_b32 a[ms_q], 0
-      .set ms_q, ms_q+1
-    .endr
     s_nop 4
     MS_WIDE_SLAB_LOADS
     s_add_u32 s84, s84, s85
     s_nop 4
     MS_WIDE_SLAB_LOADS
     s_sub_u32 s84, s84, s85
+    .set ms_q, 0
+    .rept 256
+      v_accvgpr_write_b32 a[ms_q], 0
+      .set ms_q, ms_q+1
+    .endr
     s_waitcnt vmcnt(16)
     s_barrier
     .set ms_q, 0
