@@ -1207,23 +1207,39 @@ static int small_slabs_per_split(int M, int N, int K) {
   return (slabs + s - 1) / s;
 }
 
-// 16 < M <= 64 and K a multiple of 64: the product runs as 64 x 64 tiles of the kernel whose slabs go
+// 16 < M <= 64 and K a multiple of 64: the product runs as tiles of 64 rows of the kernel whose slabs go
 // straight into LDS (it streams the weights faster than the four-wave small-M kernel: 2.9 -> 4.4 TB/s
 // at the 8B shapes), with K split so that about 768 blocks are in the grid (384 for matrices of up to
 // 16 MB, where the partial sums weigh as much as the weights: measured, 1.7 % of a batch-64 step of the
-// 0.6B shape), at most 16 splits and at least two slabs per split.
+// 0.6B shape), at most 16 splits and at least two slabs per split. Every block loads its slab of the
+// rows beside its slab of the weights, from the L2 but over the same path, so a tile of 64 columns moves
+// as many bytes of rows as of weights. Large matrices, which have columns to spare, take wider tiles:
+// 128 columns from 128 MB on (three blocks per CU), 256 columns from 400 MB on (two blocks per CU,
+// about 384 blocks). Measured at 64 rows with the weights from memory: the 8B gate/up product 47.8 ->
+// 40.9 us, the 32B gate/up 132 -> 114 and down 65 -> 57; smaller matrices lose with wider tiles (fewer
+// blocks, or more splits and partial sums).
 static bool small_runs_as_tiles(int M, int K) { return M > 16 && K % BK == 0; }
+
+static int small_tile_cols(int N, int K) {
+  const long bytes = (long)N * K * 2;
+  return bytes >= (400L << 20) ? 256 : bytes >= (128L << 20) ? 128 : 64;
+}
 
 static int tile_slabs_per_split(int N, int K) {
   const int slabs = K / BK;
-  const int cols = (N + 63) / 64;
-  const int target = (long)N * K * 2 <= (16L << 20) ? 384 : 768;
+  const int width = small_tile_cols(N, K);
+  const int cols = (N + width - 1) / width;
+  const int target = (long)N * K * 2 <= (16L << 20) || width == 256 ? 384 : 768;
   int s = (target + cols - 1) / cols;
   if (s > SMALL_MAX_SPLITS) s = SMALL_MAX_SPLITS;
   if (s > slabs / 2) s = slabs / 2;
   if (s < 1) s = 1;
   return (slabs + s - 1) / s;
 }
+
+// Columns of the tiles that a product of 17 to 64 rows (K a multiple of 64) runs as: for tests that
+// must know which instance they have reached.
+extern "C" int ms_gemm_bf16_small_tile_cols(int N, int K) { return small_tile_cols(N, K); }
 
 extern "C" int ms_gemm_bf16_small_splits(int M, int N, int K) {
   if (small_runs_as_tiles(M, K)) {
@@ -1245,8 +1261,13 @@ extern "C" int ms_gemm_bf16_small(const void* X, const void* W, float* partials,
   const int splits = ms_gemm_bf16_small_splits(M, N, K);
   if (small_runs_as_tiles(M, K) && ldx % 8 == 0) {
     const int k_per = tile_slabs_per_split(N, K) * BK;
-    const int rc = launch_dma<64, 64, BK, 2, 4>((const bf16*)X, (const bf16*)W, partials, 1, M, N, K, ldx, N, k_per,
-                                                 (size_t)M * N, splits, st);
+    const int width = small_tile_cols(N, K);
+    const int rc = width == 256   ? launch_dma<64, 256, BK, 2, 2, 1, 4>((const bf16*)X, (const bf16*)W, partials, 1, M, N, K, ldx, N,
+                                                                         k_per, (size_t)M * N, splits, st)
+                   : width == 128 ? launch_dma<64, 128, BK, 2, 3, 1, 4>((const bf16*)X, (const bf16*)W, partials, 1, M, N, K, ldx, N,
+                                                                         k_per, (size_t)M * N, splits, st)
+                                  : launch_dma<64, 64, BK, 2, 4>((const bf16*)X, (const bf16*)W, partials, 1, M, N, K, ldx, N, k_per,
+                                                                 (size_t)M * N, splits, st);
     if (rc != MS_OK) return rc;
     if (reduce) {
       if (C == nullptr || ldc < N || mode < 0 || mode > 2) return MS_BAD_ARG;

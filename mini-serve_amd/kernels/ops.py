@@ -38,6 +38,7 @@ _SIGNATURES = {
     "ms_gemm_bf16_tile_shape": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "ms_gemm_bf16_small": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gemm_bf16_small_splits": [_c_int, _c_int, _c_int],
+    "ms_gemm_bf16_small_tile_cols": [_c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],

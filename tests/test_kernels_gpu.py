@@ -287,6 +287,23 @@ def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
     assert torch.equal(rows[16][:, :9], rows[9])
 
 
+@pytest.mark.parametrize("m,n,k,cols", [(40, 16400, 4096, 128), (17, 12344, 5440, 128), (64, 51200, 4096, 256), (33, 40968, 5120, 256)])
+def test_products_of_17_to_64_rows_take_wider_tiles_on_large_matrices(ops, m, n, k, cols):
+    """From 128 MB of weights on the tiles of a 17- to 64-row product are 128 columns wide, from 400 MB on
+    256 (the library says which): other instances of the tile kernel than the 64 x 64 one that smaller
+    matrices take. N no multiple of the tile's width, an odd number of slabs, K split or not."""
+    lib = ops.library()
+    assert lib.ms_gemm_bf16_small_tile_cols(n, k) == cols, "pick other sizes for this tile width"
+    x, w = rand((m, k), BF16, 80), rand((n, k), BF16, 81, 0.05)
+    want = x.double() @ w.double().T
+    s = ops.linear(x, w, out_dtype=BF16, defer=True)
+    assert isinstance(s, ops.SplitSum) and s.splits == lib.ms_gemm_bf16_small_splits(m, n, k)
+    close(s.parts.sum(0), want, 1e-5, f"partial sums of {m}x{n}x{k}")
+    close(ops.linear(x, w, out_dtype=BF16), want, 5e-3, "finished matrix")
+    one = ops.linear(x[:1].contiguous(), w, out_dtype=F32)
+    close(one, want[:1], 1e-5, "one row of the same matrix (the small-M kernel)")
+
+
 @pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 8), (2048, 1024, 3072, 2), (300, 1000, 1100, 6), (2048, 4096, 1024, 1),
                                           (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6),
                                           (1024, 4096, 12288, 4), (768, 5120, 8192, 4), (2048, 4096, 8384, 2), (4000, 2048, 8256, 2)])
