@@ -306,12 +306,14 @@ def test_products_of_17_to_64_rows_take_wider_tiles_on_large_matrices(ops, m, n,
 
 @pytest.mark.parametrize("m,n,k,splits", [(200, 1024, 2048, 8), (2048, 1024, 3072, 2), (300, 1000, 1100, 6), (2048, 4096, 1024, 1),
                                           (96, 6144, 4096, 8), (384, 4096, 4096, 4), (130, 1024, 1088, 6),
-                                          (1024, 4096, 12288, 4), (768, 5120, 8192, 4), (2048, 4096, 8384, 2), (4000, 2048, 8256, 2)])
+                                          (1024, 4096, 12288, 4), (768, 5120, 8192, 4), (2048, 4096, 8384, 2), (4000, 2048, 8256, 2),
+                                          (500, 5120, 25600, 6)])
 def test_tile_product_splits_k_when_tiles_are_few(ops, m, n, k, splits):
     """The last four have 256 and more tiles of 128 x 128 already: above 512 rows the splits follow the
     predicted time (a long K in parts makes 256 x 256 tiles enough to give every CU one), not the tile
     count alone. The very last two have a last split that is one slab shorter than the others, with an
-    odd and an even number of slabs."""
+    odd and an even number of slabs; the last one is a large matrix at under 512 rows, which takes many
+    short splits for the same reason."""
     x, w = rand((m, k), BF16, 60), rand((n, k), BF16, 61, 0.05)
     want = x.double() @ w.double().T
     resid = rand((m, n), F32, 62)
