@@ -1214,7 +1214,7 @@ static int small_slabs_per_split(int M, int N, int K) {
 // 0.6B shape), at most 16 splits and at least two slabs per split. Every block loads its slab of the
 // rows beside its slab of the weights, from the L2 but over the same path, so a tile of 64 columns moves
 // as many bytes of rows as of weights. Large matrices, which have columns to spare, take wider tiles:
-// 128 columns from 256 MB on (three blocks per CU), 256 columns from 400 MB on (two blocks per CU,
+// 128 columns from 224 MB on (three blocks per CU), 256 columns from 400 MB on (two blocks per CU,
 // about 384 blocks). Measured at 64 rows with the weights from memory: the 32B gate/up product 132 ->
 // 114 us and down 65 -> 57, a decode step of the 32B shape at batch 64 8.5 % faster; smaller matrices
 // lose with wider tiles (fewer blocks, or more splits and partial sums), and the 8B gate/up product
@@ -1223,7 +1223,7 @@ static bool small_runs_as_tiles(int M, int K) { return M > 16 && K % BK == 0; }
 
 static int small_tile_cols(int N, int K) {
   const long bytes = (long)N * K * 2;
-  return bytes >= (400L << 20) ? 256 : bytes >= (256L << 20) ? 128 : 64;
+  return bytes >= (400L << 20) ? 256 : bytes >= (224L << 20) ? 128 : 64;
 }
 
 static int tile_slabs_per_split(int N, int K) {

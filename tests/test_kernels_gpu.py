@@ -289,7 +289,7 @@ def test_small_product_with_shared_rows_on_large_matrices(ops, n, k):
 
 @pytest.mark.parametrize("m,n,k,cols", [(40, 32776, 4096, 128), (17, 24680, 5440, 128), (64, 51200, 4096, 256), (33, 40968, 5120, 256)])
 def test_products_of_17_to_64_rows_take_wider_tiles_on_large_matrices(ops, m, n, k, cols):
-    """From 256 MB of weights on the tiles of a 17- to 64-row product are 128 columns wide, from 400 MB on
+    """From 224 MB of weights on the tiles of a 17- to 64-row product are 128 columns wide, from 400 MB on
     256 (the library says which): other instances of the tile kernel than the 64 x 64 one that smaller
     matrices take. N no multiple of the tile's width, an odd number of slabs, K split or not."""
     lib = ops.library()
