@@ -494,7 +494,7 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
 
 // ---------------------------------------------------------------------------------------------
 // 256 x 256 tile with four waves, each with a wave tile of 128 x 128: 16 fragment reads for 64
-// products (the eight-wave tile above reads 12 for 32), so that fragment reads and the loads into LDS
+// products (eight waves with wave tiles of 64 x 128, which the kernel above can be built with, read 12 for 32), so that fragment reads and the loads into LDS
 // together keep the LDS busy three quarters of the time the products take instead of all of it. The 256
 // accumulator registers of a lane are all the AGPRs there are, and one wave per SIMD has nobody to
 // cover its waits, so registers and instruction order of the loop over K are written out: the loop is
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(WR * WC * WAVE, BLOCKS_PER_CU) void gemm_bf16_dma_k
 // AGPRs alone: it has no use for them here (no matrix builtins, 96 VGPRs of its own and nothing spilled:
 // the kernel's scratch size is 0), and every statement names all of them as clobbered.
 // One block per CU stays for the whole product and takes tiles in turn. Measured at 8192^3, sustained, at
-// the socket's power limit: 1,500 TFLOP/s against 1,260 of the eight-wave tile and 1,620 of the vendor
+// the socket's power limit: 1,500 TFLOP/s against 1,260 of that eight-wave tile and 1,620 of the vendor
 // library; at 2,048 x 24,576 x 4,096 1,506 against 1,175 and 1,530.
 
 // Accumulator fragment F of the wide tile's loop, out of the AGPRs.
