@@ -228,6 +228,60 @@ def test_gemm_bf16_large_tiles(ops, m, n, k, tile):
     close(acc, before.double() + want, 1e-5, "gemm bf16 accumulate")
 
 
+def _wide_tile_draws(seed):
+    """Sizes drawn at random (a fixed seed): rows and columns with ragged edges, K from two slabs on, plain and gated."""
+    import random
+    rng = random.Random(seed)
+    while True:
+        m = rng.choice([rng.randint(257, 5000), rng.choice([512, 1024, 2048, 4096])])
+        n = rng.choice([rng.randint(32, 800) * 8, rng.choice([4096, 5120, 6144])])
+        k = rng.choice([128, 192, 256, 320, 1024, 2048, 4160]) if rng.random() < 0.7 else rng.randint(2, 60) * 64
+        gated = rng.random() < 0.3
+        yield m, (n // 32 * 32 if gated else n), k, gated
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_wide_tile_at_random_sizes(ops, seed):
+    """The four-wave 256 x 256 tile, whose loop is written in assembly, at sizes nobody chose: every output
+    form (bfloat16, float32, added into a float32 matrix, partial sums of a split K, gated with both
+    activations) against float64, and twice for equal bits (a tile taken by another block, in another turn,
+    must give the same)."""
+    lib = ops.library()
+    done = 0
+    for tries, (m, n, k, gated) in enumerate(_wide_tile_draws(seed)):
+        if done == 8 or tries == 4000:
+            break
+        if m * n > 24e6 or (m + n) * k > 60e6:
+            continue
+        splits = 1 if gated else lib.ms_gemm_bf16_tile_splits(m, n, k)
+        if ops.tile_shape(m, n, k, splits, gated) != (256, 256):
+            continue
+        done += 1
+        what = f"{m}x{n}x{k} splits {splits} gated {gated}"
+        x, w = rand((m, k), BF16, 300 + done), rand((n, k), BF16, 400 + done, 0.05)
+        want = x.double() @ w.double().T
+        if gated:
+            pairs = want.view(m, n // 32, 2, 16)
+            g, u = pairs[:, :, 0].reshape(m, n // 2), pairs[:, :, 1].reshape(m, n // 2)
+            for act in ("silu", "gelu_tanh"):
+                a = ops.gated_linear(x, w, act, out_dtype=BF16, block=ops.GATE_BLOCK)
+                close(a, activation(act, g) * u, 8e-3, f"{what} {act}")
+                assert torch.equal(a, ops.gated_linear(x, w, act, out_dtype=BF16, block=ops.GATE_BLOCK)), what
+            continue
+        a = ops.linear(x, w, out_dtype=BF16)
+        close(a, want, 5e-3, f"{what} -> bf16")
+        assert torch.equal(a, ops.linear(x, w, out_dtype=BF16)), what
+        close(ops.linear(x, w, out_dtype=F32), want, 1e-5, f"{what} -> f32")
+        acc = rand((m, n), F32, 500 + done)
+        before = acc.clone()
+        pend = ops.linear(x, w, accumulate_into=acc, defer=True)
+        if pend is not None:
+            assert pend.splits == splits, what
+            ops.add_pending(acc, pend)
+        close(acc.double() - before.double(), want, 1e-5, f"{what} accumulate")
+    assert done == 8, "the draw no longer reaches the 256 x 256 tile often enough: widen it"
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 40, 64])
 def test_pending_sums_feed_their_consumers(ops, m):
     """The small-M product may leave partial sums for the next kernel to add: every consumer of such
